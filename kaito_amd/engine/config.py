@@ -101,6 +101,9 @@ class ModelConfig:
     n_group: int = 1                     # expert groups (V3: 8)
     topk_group: int = 1                  # groups kept per token (V3: 4)
     n_shared_experts: int = 0            # always-on experts (width = n*moe_ie)
+    # width of the always-on expert when it is not a multiple of the routed
+    # experts' (overrides n_shared_experts)
+    moe_shared_intermediate_size: int = 0
     first_k_dense: int = 0               # leading dense (non-MoE) layers
     # ---- YaRN rope scaling (DeepSeek long-context) ----------------------
     rope_scaling_type: str = ""          # "" | "yarn"
@@ -131,6 +134,9 @@ class ModelConfig:
     # the residual stream is held and summed in f32 (norms read it in
     # f32); sub-layers see its rounding to `dtype`
     residual_fp32: bool = False
+    # hashed bigram table added to the token embedding
+    # (models/hybrid_config.py BigramSpec); None = token embedding only
+    bigram: Optional[object] = None
 
     @classmethod
     def from_hf_config(cls, cfg: dict, name: str = "") -> "ModelConfig":

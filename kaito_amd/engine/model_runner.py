@@ -230,6 +230,7 @@ class ModelRunner:
                 [c.start for c in chunks], dtype=torch.int32, device=dev)
             meta.token_seq = torch.tensor(seq_of, dtype=torch.int32,
                                           device=dev)
+            meta.ctx_lens = [c.start + c.length for c in chunks]
             if self.is_gpu and meta.max_seqlen >= 8:
                 # prompt portions: tile the chunks for the MFMA attention
                 # kernel (a step of single tokens keeps the decode kernel)

@@ -69,9 +69,17 @@ class HybridStackBase(nn.Module):
         """No position table: rotations, where a design has them, are
         computed from the position inside the kernels."""
 
+    def stack_state(self, num_slots, device) -> Dict:
+        """Per-sequence state that belongs to the stack rather than to a
+        layer (slot-indexed tensors); handed to forward() as the entry
+        after the layers' caches. Default: none."""
+        return {}
+
     def cache_bytes(self, block_size: int):
         """(bytes per KV page, bytes per state slot) over all layers."""
-        page = slot = 0
+        page = 0
+        slot = sum(t.element_size() * t[0].numel()
+                   for t in self.stack_state(1, "cpu").values())
         for layer in self.layers:
             for m in layer.mixers():
                 p, s = m.cache_bytes(block_size)
@@ -82,7 +90,8 @@ class HybridStackBase(nn.Module):
     def alloc_caches(self, num_blocks, block_size, num_slots,
                      device) -> List[Dict]:
         return [layer.alloc_cache(num_blocks, block_size, num_slots, device)
-                for layer in self.layers]
+                for layer in self.layers] \
+            + [self.stack_state(num_slots, device)]
 
     def compute_logits(self, hidden: torch.Tensor) -> torch.Tensor:
         """hidden: rows of the f32 residual stream → f32 logits."""

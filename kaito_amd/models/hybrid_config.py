@@ -1,6 +1,6 @@
-"""Per-layer specifications for hybrid stacks (recurrent + windowed
-attention layers mixed in one model) and the config.json readers of the
-Gurapel and Pokulorn designs.
+"""Per-layer specifications for hybrid stacks (recurrent, windowed and
+latent attention layers mixed in one model) and the config.json readers of
+the Gurapel, Pokulorn and Munerax designs.
 
 A homogeneous model is described by the flat ModelConfig fields; a hybrid
 one additionally carries `layer_specs`, one LayerSpec per layer, each
@@ -59,9 +59,23 @@ class RGLRUSpec:
 
 @dataclass(frozen=True)
 class MoESpec:
+    """Routed feed-forward. `routing`: "topk_softmax" (top-k of the
+    logits, softmax over the chosen ones) or "sigmoid_groups" (sigmoid
+    scores; experts form `groups` equal groups of neighbours, a group
+    scores the sum of its two best experts, only the `keep_groups` best
+    groups are eligible; weights are the chosen scores times `scale`, not
+    renormalised). `act`: "silu_glu" (gated experts) or "relu2" (ungated,
+    squared relu). `shared_ff` > 0 adds an always-on expert of that width
+    and the same form."""
     experts: int
     top: int
     ff: int
+    routing: str = "topk_softmax"
+    act: str = "silu_glu"
+    groups: int = 1
+    keep_groups: int = 1
+    scale: float = 1.0
+    shared_ff: int = 0
 
 
 @dataclass(frozen=True)
@@ -156,7 +170,47 @@ class DenseFFSpec:
 
 
 @dataclass(frozen=True)
+class LatentAttnSpec:
+    """Softmax attention whose keys and values are up-projections of one
+    low-rank latent per token: the cache holds the RMS-normed latent
+    (`kv_rank`) and one rotated key part (`rot_dim`) shared by all heads.
+    Per head, `dim` unrotated plus `rot_dim` rotated query/key dimensions
+    and `vdim` value dimensions. Options: a per-head sink in the softmax
+    denominator, a per-head sigmoid output gate, and `kv_from` = index of
+    an earlier layer whose cached latent and rotated key this layer
+    reads instead of projecting its own."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    kv_rank: int
+    scale: float
+    rot: Optional[RotarySpec] = None
+    sink: bool = False
+    gate: bool = False
+    kv_from: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class GeluGLUSpec:
+    """Gated feed-forward down(gelu_tanh(gate)·up)."""
+    ff: int
+
+
+@dataclass(frozen=True)
+class BigramSpec:
+    """Hashed bigram embedding added to the token embedding: row
+    (previous·mul_prev + token·mul_cur) mod buckets of a [buckets + 1,
+    width] table; a sequence's first token takes the last row."""
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+
+
+@dataclass(frozen=True)
 class LayerSpec:
+    # Munerax — "latent_attention": LatentAttnSpec, with `glu` (dense) or
+    # `moe` as its feed-forward.
     # Gurapel — "delta": one DeltaRuleSpec; "parallel": WindowAttnSpec
     # beside RGLRUSpec, outputs normed and averaged.
     # Pokulorn — "mlstm": MLSTMSpec; "attention": RotaryAttnSpec;
@@ -172,6 +226,8 @@ class LayerSpec:
     ssd: Optional[SSDSpec] = None
     dense: Optional[DenseFFSpec] = None
     branch_scales: Tuple[float, float] = (1.0, 1.0)
+    latent: Optional[LatentAttnSpec] = None
+    glu: Optional[GeluGLUSpec] = None
 
 
 def _moe_spec(m) -> Optional[MoESpec]:
@@ -251,9 +307,12 @@ def layer_moe_config(cfg: ModelConfig, moe: MoESpec) -> ModelConfig:
         ff = (ff + 63) // 64 * 64
     return dataclasses.replace(
         cfg, num_experts=moe.experts, num_experts_per_tok=moe.top,
-        moe_intermediate_size=ff, moe_routing="topk_softmax",
-        moe_act="silu", moe_bias=False, n_shared_experts=0,
-        moe_router_fp32=True)
+        moe_intermediate_size=ff, moe_routing=moe.routing,
+        moe_act="silu" if moe.act == "silu_glu" else moe.act,
+        moe_bias=False, n_shared_experts=0,
+        moe_shared_intermediate_size=moe.shared_ff, n_group=moe.groups,
+        topk_group=moe.keep_groups, moe_norm_topk=False,
+        routed_scaling_factor=moe.scale, moe_router_fp32=True)
 
 
 # ---- Pokulorn ---------------------------------------------------------------
@@ -341,3 +400,89 @@ def pokulorn_model_config(cfg: dict, name: str = "",
                                  POKULORN_DEFAULT_MAX_POSITION)),
         rms_eps=float(cfg["norm"]["eps"]),
         residual_fp32=True, dtype=dtype)
+
+
+# ---- Munerax ------------------------------------------------------------------
+
+def _munerax_ff(m):
+    """config `mlp` entry → (GeluGLUSpec | None, MoESpec | None)."""
+    if m is None:
+        return None, None
+    kind = m.get("kind", "dense")
+    if kind == "dense":
+        return GeluGLUSpec(ff=int(m["ff"])), None
+    if kind != "moe":
+        raise ValueError(f"unsupported feed-forward kind {kind!r}")
+    r = m["router"]
+    g = r.get("groups") or {}
+    shared = m.get("shared") or {}
+    return None, MoESpec(
+        experts=int(r["experts"]), top=int(r["top"]),
+        ff=int(m["expert"]["ff"]), routing="sigmoid_groups", act="relu2",
+        groups=int(g.get("count", 1)), keep_groups=int(g.get("keep", 1)),
+        scale=float(r.get("scale", 1.0)), shared_ff=int(shared.get("ff", 0)))
+
+
+def _munerax_layer(entry: dict, index: int, layers: list) -> LayerSpec:
+    kind, mx = entry["type"], entry["mixer"]
+    if kind != "latent_attention":
+        raise ValueError(f"unknown layer type {kind!r}")
+    rot = mx["rot"]
+    if int(rot["dims"]) != int(mx["rot_dim"]):
+        raise ValueError("the rotated key part is rotated whole")
+    src = mx.get("kv_from")
+    if src is not None:
+        src = int(src)
+        other = layers[src]["mixer"] if 0 <= src < index else None
+        if other is None or other.get("kv_from") is not None:
+            raise ValueError(f"layer {index}: kv_from must name an earlier "
+                             "layer with a down-projection of its own")
+        for k in ("kv_rank", "rot_dim"):
+            if int(other[k]) != int(mx[k]):
+                raise ValueError(f"layer {index}: {k} differs from layer "
+                                 f"{src}, whose cache it reads")
+    glu, moe = _munerax_ff(entry.get("mlp"))
+    return LayerSpec(kind, latent=LatentAttnSpec(
+        heads=int(mx["heads"]), dim=int(mx["dim"]),
+        rot_dim=int(mx["rot_dim"]), vdim=int(mx["vdim"]),
+        kv_rank=int(mx["kv_rank"]), scale=float(mx["scale"]),
+        rot=RotarySpec(dims=int(rot["dims"]), base=float(rot["base"])),
+        sink=True, gate=True, kv_from=src), glu=glu, moe=moe)
+
+
+def is_munerax_config(cfg: dict) -> bool:
+    return cfg.get("architecture") == "Munerax"
+
+
+def munerax_model_config(cfg: dict, name: str = "",
+                         dtype: torch.dtype = torch.bfloat16) -> ModelConfig:
+    """config.json of a Munerax checkpoint → ModelConfig (every size, the
+    layer order and every per-model constant come from the file). The
+    design has no position table, so its length limit is the engine's."""
+    layers = cfg["layers"]
+    specs: Tuple[LayerSpec, ...] = tuple(
+        _munerax_layer(e, i, layers) for i, e in enumerate(layers))
+    width = int(cfg["width"])
+    att = specs[0].latent
+    moe = next((s.moe for s in specs if s.moe is not None), None)
+    glu = next((s.glu for s in specs if s.glu is not None), None)
+    emb = cfg["embedding"]
+    bg = emb.get("bigram")
+    return ModelConfig(
+        name=name or "munerax", arch="munerax", layer_specs=specs,
+        hidden_size=width, num_layers=len(specs),
+        num_heads=att.heads, num_kv_heads=1,
+        head_dim=att.dim + att.rot_dim,
+        intermediate_size=glu.ff if glu else (moe.ff if moe else width),
+        vocab_size=int(cfg["vocab"]),
+        max_position=int(cfg.get("max_positions",
+                                 POKULORN_DEFAULT_MAX_POSITION)),
+        rms_eps=float(cfg["norm"]["eps"]),
+        embed_scale=float(emb.get("scale", 1.0)),
+        bigram=BigramSpec(buckets=int(bg["buckets"]),
+                          mul_prev=int(bg["mul_prev"]),
+                          mul_cur=int(bg["mul_cur"])) if bg else None,
+        tie_word_embeddings=True, residual_fp32=True,
+        num_experts=moe.experts if moe else 0,
+        num_experts_per_tok=moe.top if moe else 0,
+        moe_intermediate_size=moe.ff if moe else 0, dtype=dtype)

@@ -47,6 +47,9 @@ class AttnMetadata:
     # 64-row query tiles of the chunks (steps that hold prompt portions)
     tile_seq: Optional[torch.Tensor] = None      # [tiles] int32
     tile_qbase: Optional[torch.Tensor] = None    # [tiles] int32
+    # host copy of each chunk's context length after the step (start +
+    # chunk length), for ops that size step-local buffers by it
+    ctx_lens: Optional[list] = None
     # values one layer of a step leaves for later layers of the same step
     # (the model's forward sets an empty dict)
     layer_shared: Optional[dict] = None

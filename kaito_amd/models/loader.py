@@ -28,6 +28,8 @@ def load_safetensors_weights(model, path: str,
         return load_gurapel_weights(model, path)
     if getattr(model.cfg, "arch", "llama") == "pokulorn":
         return load_pokulorn_weights(model, path)
+    if getattr(model.cfg, "arch", "llama") == "munerax":
+        return load_munerax_weights(model, path)
     from safetensors.torch import safe_open
 
     cfg = model.cfg
@@ -430,4 +432,56 @@ def load_pokulorn_weights(model, path: str) -> None:
             put(layer.mlp.gate_up, torch.cat(
                 [get(fp + "gate"), get(fp + "up")], 0))
             put(layer.mlp.down, get(fp + "down"))
+    ck.warn_unused()
+
+
+def load_munerax_weights(model, path: str) -> None:
+    """Munerax checkpoint (flat tensor names, `l<i>.` per layer, mixer
+    tensors under `.mix.`, feed-forward under `.mlp.`, linear weights
+    [out, in]) → MuneraxForCausalLM. Fuses each mixer's input projections
+    (query, gate, latent down-projection), stacks the experts (zero-filled
+    up to the kernels' tile width) and widens per-channel tensors to f32."""
+    ck = _FlatCheckpoint(path)
+    get, put = ck.get, ck.put
+    put(model.embed_tokens.weight, get("embed"))
+    if model.bigram is not None:
+        put(model.bigram, get("bigram"))
+    put(model.norm, get("final.norm").float())
+    for i, layer in enumerate(model.layers):
+        pre = f"l{i}."
+        a, ap = layer.attn, pre + "mix."
+        s = a.spec
+        put(layer.norm1, get(pre + "norm1").float())
+        names = ("q",) + (("g",) if s.gate else ()) \
+            + (("dkv",) if a.own_kv else ())
+        put(a.in_proj, torch.cat([get(ap + n) for n in names], 0))
+        if a.own_kv:
+            put(a.kv_norm, get(ap + "dkv.norm").float())
+        put(a.w_uk, get(ap + "uk"))
+        put(a.w_uv, get(ap + "uv"))
+        if s.sink:
+            put(a.sinks, get(ap + "sink").float())
+        put(a.o_proj, get(ap + "o"))
+        if layer.mlp is None:
+            continue
+        fp = pre + "mlp."
+        put(layer.norm2, get(pre + "norm2").float())
+        if layer.spec.glu is not None:
+            put(layer.mlp.gate_up, torch.cat(
+                [get(fp + "gate"), get(fp + "up")], 0))
+            put(layer.mlp.down, get(fp + "down"))
+            continue
+        mlp = layer.mlp
+        put(mlp.gate, get(fp + "router").float())
+        with torch.no_grad():
+            mlp.w_gate_up.zero_()
+            mlp.w_down.zero_()
+            for e in range(mlp.num_experts):
+                u, d = get(f"{fp}e{e}.up"), get(f"{fp}e{e}.down")
+                ff = u.shape[0]
+                mlp.w_gate_up[e, :ff].copy_(u.to(mlp.w_gate_up.dtype))
+                mlp.w_down[e, :, :ff].copy_(d.to(mlp.w_down.dtype))
+        if mlp.w_shared_gate_up is not None:
+            put(mlp.w_shared_gate_up, get(fp + "shared.up"))
+            put(mlp.w_shared_down, get(fp + "shared.down"))
     ck.warn_unused()

@@ -2,7 +2,9 @@
 recurrence, matrix-memory (mLSTM) recurrence, scalar-decay selective
 state space, and softmax attention over the paged cache in two flavours
 (distance penalty without rotation; convolutions + rotation + window
-with kept first tokens + sink). Each is a self-contained module
+with kept first tokens + sink), and latent attention (one low-rank
+latent per token in the cache, optionally borrowed from an earlier
+layer). Each is a self-contained module
 parameterised by its spec (models/hybrid_config.py), so a design picks
 and combines them freely.
 
@@ -30,7 +32,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .. import ops
-from .hybrid_config import (DeltaRuleSpec, DenseFFSpec, MLSTMSpec, RGLRUSpec,
+from .hybrid_config import (DeltaRuleSpec, DenseFFSpec, GeluGLUSpec,
+                            LatentAttnSpec, MLSTMSpec, RGLRUSpec,
                             RotaryAttnSpec, SSDSpec, WindowAttnSpec)
 
 
@@ -454,3 +457,134 @@ class ClampedGLU(nn.Module):
         a = ops.clamped_glu(F.linear(x, self.gate_up), self.spec.limit,
                             self.spec.alpha)
         return F.linear(a, self.down)
+
+
+class LatentAttention(nn.Module):
+    """Softmax attention over a paged cache of low-rank latents. Per token
+    the cache holds c = rms(W_dkv x)[:rank]·w and one rotated key part of
+    `rot_dim` dims shared by all heads; head h's key is [W_uk,h c | rotated
+    part] and its value W_uv,h c. Queries carry `dim` unrotated and
+    `rot_dim` rotated dims per head. Options: per-head sink in the softmax
+    denominator, per-head sigmoid output gate read from the mixer input.
+    With spec.kv_from set the mixer has no down-projection and reads the
+    cache of the layer it names (the caller passes that layer's cache).
+
+    Two equivalent evaluations (key and value are linear in c):
+      * latent form — the unrotated query is folded through W_uk
+        (q_c = W_uk,hᵀ q), scores are q_c·c + q_rot·k_rot, the weighted sum
+        runs over c and W_uv is applied to the result. One pass over the
+        cache serves every head; used for single tokens and in f32.
+      * expanded form — for prompt portions in bf16 the latents of the
+        step's sequences are gathered, up-projected to per-head keys and
+        values in a step-local paged scratch, and the MFMA attention
+        kernel of the window mixers runs on it (fewer flops per score:
+        dim + rot_dim instead of rank + rot_dim)."""
+
+    def __init__(self, hidden: int, spec: LatentAttnSpec, dtype,
+                 norm_eps: float):
+        super().__init__()
+        self.spec, self.dtype, self.norm_eps = spec, dtype, norm_eps
+        s = spec
+        assert s.rot is not None and s.rot.dims == s.rot_dim \
+            and s.rot_dim % 2 == 0
+        self.own_kv = s.kv_from is None
+        self.q_size = s.heads * (s.dim + s.rot_dim)
+        self.g_size = s.heads if s.gate else 0
+        self.row = s.kv_rank + s.rot_dim
+        # fused input projection, rows [q | gate | latent + rotated key]
+        self.in_proj = _p(self.q_size + self.g_size
+                          + (self.row if self.own_kv else 0), hidden,
+                          dtype=dtype)
+        self.kv_norm = _p(s.kv_rank, dtype=torch.float32) \
+            if self.own_kv else None
+        self.w_uk = _p(s.heads * s.dim, s.kv_rank, dtype=dtype)
+        self.w_uv = _p(s.heads * s.vdim, s.kv_rank, dtype=dtype)
+        freq, _ = s.rot.frequencies()
+        self.register_buffer("inv_freq", torch.tensor(
+            freq, dtype=torch.float64).float(), persistent=False)
+        self.sinks = _p(s.heads, dtype=torch.float32) if s.sink else None
+        self.o_proj = _p(hidden, s.heads * s.vdim, dtype=dtype)
+
+    def alloc_cache(self, num_blocks, block_size, num_slots, device) -> Dict:
+        if not self.own_kv:
+            return {}
+        return {"kv": torch.zeros(num_blocks, block_size, self.row,
+                                  dtype=self.dtype, device=device)}
+
+    def cache_bytes(self, block_size: int):
+        if not self.own_kv:
+            return 0, 0
+        esz = torch.empty(0, dtype=self.dtype).element_size()
+        return block_size * self.row * esz, 0
+
+    def _expanded_ok(self, x, meta) -> bool:
+        s = self.spec
+        return (x.is_cuda and x.dtype == torch.bfloat16
+                and meta.tile_seq is not None
+                and meta.ctx_lens is not None
+                and s.dim + s.rot_dim <= max(ops.WINDOW_MFMA_SIZES)
+                and s.vdim <= max(ops.WINDOW_MFMA_VSIZES))
+
+    def forward(self, x, positions, cache, meta):
+        s = self.spec
+        T, H, D = x.size(0), s.heads, s.dim
+        p = F.linear(x, self.in_proj)
+        q = p[:, :self.q_size].unflatten(-1, (H, D + s.rot_dim))
+        dkv = p[:, self.q_size + self.g_size:] if self.own_kv else None
+        kv = cache["kv"]
+        qr = ops.latent_rope_cache_write(
+            q, dkv, self.kv_norm, self.norm_eps, kv, meta.slot_mapping,
+            positions, self.inv_freq, D)
+        if self._expanded_ok(x, meta):
+            o = self._expanded(qr, kv, meta)
+        else:
+            qc = torch.bmm(qr[..., :D].transpose(0, 1),
+                           self.w_uk.view(H, D, s.kv_rank))     # [H, T, r]
+            qf = torch.cat([qc.transpose(0, 1), qr[..., D:]], -1)
+            oc = ops.latent_attention(qf, kv, meta.block_tables,
+                                      meta.token_seq, positions, s.scale,
+                                      s.kv_rank, self.sinks)     # [T, H, r]
+            o = torch.bmm(oc.transpose(0, 1),
+                          self.w_uv.view(H, s.vdim, s.kv_rank)
+                          .transpose(1, 2)).transpose(0, 1)
+        o = o.reshape(T, H * s.vdim)
+        if s.gate:
+            o = ops.sigmoid_mul(o, p[:, self.q_size:self.q_size + H])
+        return F.linear(o, self.o_proj)
+
+    def _expanded(self, qr, kv, meta):
+        """Prompt portions (bf16): per-head keys and values of the step's
+        sequences in a step-local paged scratch, then the MFMA kernel."""
+        s = self.spec
+        H, D, R, V = s.heads, s.dim, s.rot_dim, s.vdim
+        Dp = next(d for d in ops.WINDOW_MFMA_SIZES if d >= D + R)
+        Vp = next(v for v in ops.WINDOW_MFMA_VSIZES if v >= V)
+        lat, tables = ops.latent_gather(kv, meta.block_tables, meta.ctx_lens)
+        k_s, v_s = ops.latent_expand(
+            F.linear(lat[:, :s.kv_rank], self.w_uk),
+            F.linear(lat[:, :s.kv_rank], self.w_uv), lat, H, D, V, Dp, Vp,
+            kv.size(1))
+        T = qr.size(0)
+        if Dp != D + R:
+            qp = qr.new_zeros(T, H, Dp)
+            qp[..., :D + R] = qr
+        else:
+            qp = qr
+        o = ops.window_attention(
+            qp, k_s, v_s, tables, meta.token_seq, None, s.scale,
+            tiles=(meta.tile_seq, meta.tile_qbase, meta.cu_seqlens,
+                   meta.seq_starts), sinks=self.sinks)
+        return o[..., :V]
+
+
+class GeluGLU(nn.Module):
+    """Dense gated feed-forward down(gelu_tanh(gate x) · up x)."""
+
+    def __init__(self, hidden: int, spec: GeluGLUSpec, dtype):
+        super().__init__()
+        self.spec = spec
+        self.gate_up = _p(2 * spec.ff, hidden, dtype=dtype)   # [gate | up]
+        self.down = _p(hidden, spec.ff, dtype=dtype)
+
+    def forward(self, x):
+        return F.linear(ops.gelu_glu(F.linear(x, self.gate_up)), self.down)

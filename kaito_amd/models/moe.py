@@ -56,10 +56,16 @@ class MoEMLP(nn.Module):
         self.gate = nn.Parameter(
             torch.empty(e, h, dtype=torch.float32 if cfg.moe_router_fp32
                         else cfg.dtype), requires_grad=False)
+        # "relu2": ungated experts down(relu(up x)^2); everything else is
+        # gated (act(gate x) * up x)
+        self.gated = cfg.moe_act != "relu2"
+        rows = 2 if self.gated else 1
         # stacked expert weights (local shard):
-        # [E_l, 2*IE_l, h] (gate|up) and [E_l, h, IE_l]
+        # [E_l, 2*IE_l, h] (gate|up; ungated: [E_l, IE_l, h], up only)
+        # and [E_l, h, IE_l]
         self.w_gate_up = nn.Parameter(
-            torch.empty(self.e_local, 2 * self.ie_local, h, dtype=cfg.dtype),
+            torch.empty(self.e_local, rows * self.ie_local, h,
+                        dtype=cfg.dtype),
             requires_grad=False)
         self.w_down = nn.Parameter(
             torch.empty(self.e_local, h, self.ie_local, dtype=cfg.dtype),
@@ -74,7 +80,7 @@ class MoEMLP(nn.Module):
         else:
             self.b_gate_up = None
             self.b_down = None
-        self.act_mode = 1 if cfg.moe_act == "swiglu_oai" else 0
+        self.act_mode = {"swiglu_oai": 1, "relu2": 2}.get(cfg.moe_act, 0)
         # deepseek-v3 noaux_tc routing: per-expert selection bias
         if cfg.moe_routing == "noaux_tc":
             self.e_score_correction_bias = nn.Parameter(
@@ -82,12 +88,13 @@ class MoEMLP(nn.Module):
         # deepseek shared experts: always-on dense SwiGLU of width
         # n_shared * moe_ie, IE-sharded over TP; its down output is a
         # TP-partial like the routed output, so both ride ONE all-reduce
-        if cfg.n_shared_experts > 0:
-            sie = cfg.n_shared_experts * ie
+        if cfg.n_shared_experts > 0 or cfg.moe_shared_intermediate_size > 0:
+            sie = cfg.moe_shared_intermediate_size \
+                or cfg.n_shared_experts * ie
             assert tp == 1 or sie % tp == 0, (sie, tp)
             self.sie_local = sie // tp
             self.w_shared_gate_up = nn.Parameter(
-                torch.empty(2 * self.sie_local, h, dtype=cfg.dtype),
+                torch.empty(rows * self.sie_local, h, dtype=cfg.dtype),
                 requires_grad=False)
             self.w_shared_down = nn.Parameter(
                 torch.empty(h, self.sie_local, dtype=cfg.dtype),
@@ -104,11 +111,13 @@ class MoEMLP(nn.Module):
             logits = torch.nn.functional.linear(x.float(), self.gate)
         else:
             logits = torch.nn.functional.linear(x, self.gate)  # [T, E]
-        if cfg.moe_routing == "noaux_tc":
+        if cfg.moe_routing in ("noaux_tc", "sigmoid_groups"):
             # deepseek-v3: sigmoid scores; SELECTION uses scores+bias with
-            # group-limited top-k; WEIGHTS are the original sigmoid scores
+            # group-limited top-k; WEIGHTS are the original sigmoid scores.
+            # "sigmoid_groups" is the same without a selection bias.
             scores = torch.sigmoid(logits.float())
-            sel = scores + self.e_score_correction_bias
+            sel = scores + self.e_score_correction_bias \
+                if cfg.moe_routing == "noaux_tc" else scores
             if cfg.n_group > 1:
                 gs = sel.view(T, cfg.n_group, -1)
                 group_score = gs.topk(min(2, gs.size(-1)), dim=-1)[0].sum(-1)
@@ -164,7 +173,8 @@ class MoEMLP(nn.Module):
         T, H = x.shape
         sorted_tok, gates, offsets = self._route(x)
         fused_shapes = (x.is_cuda and x.dtype == torch.bfloat16
-                        and H % 64 == 0 and self.ie_local % 64 == 0)
+                        and H % 64 == 0 and self.ie_local % 64 == 0
+                        and self.gated)
         # under hipGraph capture the fused kernels are mandatory (the
         # per-expert loop reads segment sizes on the host): deepseek k=6
         # crosses TK=4096 at decode bs>682 and measured 30.9k vs timeout
@@ -177,7 +187,8 @@ class MoEMLP(nn.Module):
         if self.w_shared_gate_up is not None:   # deepseek shared experts
             h1 = torch.nn.functional.linear(x, self.w_shared_gate_up)
             out = out + torch.nn.functional.linear(
-                ops.silu_and_mul(h1), self.w_shared_down)
+                ops.silu_and_mul(h1) if self.gated else ops.relu2(h1),
+                self.w_shared_down)
         if get_state().tp_size > 1:
             out = tp_all_reduce(out)
         return out
@@ -217,7 +228,9 @@ class MoEMLP(nn.Module):
             h1 = torch.nn.functional.linear(
                 xs, self.w_gate_up[le],
                 self.b_gate_up[le] if self.b_gate_up is not None else None)
-            if self.act_mode == 1:
+            if self.act_mode == 2:
+                act = ops.relu2(h1)
+            elif self.act_mode == 1:
                 g, u = h1.float().chunk(2, dim=-1)
                 g = g.clamp(max=7.0)
                 u = u.clamp(-7.0, 7.0)

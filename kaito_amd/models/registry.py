@@ -25,6 +25,7 @@ MODEL_CLASSES: Dict[str, str] = {
     "llama": "kaito_amd.models.llama:LlamaForCausalLM",
     "gurapel": "kaito_amd.models.gurapel:GurapelForCausalLM",
     "pokulorn": "kaito_amd.models.pokulorn:PokulornForCausalLM",
+    "munerax": "kaito_amd.models.munerax:MuneraxForCausalLM",
 }
 
 
@@ -43,12 +44,15 @@ def config_from_checkpoint(cfg_json: dict, name: str = "",
     """config.json dict → ModelConfig, choosing the reader by the file's
     own architecture tag."""
     from .hybrid_config import (gurapel_model_config, is_gurapel_config,
-                                is_pokulorn_config, pokulorn_model_config)
+                                is_munerax_config, is_pokulorn_config,
+                                munerax_model_config, pokulorn_model_config)
     kw = {"dtype": dtype} if dtype is not None else {}
     if is_gurapel_config(cfg_json):
         return gurapel_model_config(cfg_json, name=name, **kw)
     if is_pokulorn_config(cfg_json):
         return pokulorn_model_config(cfg_json, name=name, **kw)
+    if is_munerax_config(cfg_json):
+        return munerax_model_config(cfg_json, name=name, **kw)
     cfg = ModelConfig.from_hf_config(cfg_json, name=name)
     if dtype is not None:
         import dataclasses
@@ -403,3 +407,35 @@ def _tiny_pokulorn() -> ModelConfig:
 
 
 register(_tiny_pokulorn())
+
+
+def _tiny_munerax() -> ModelConfig:
+    """A small latent-attention stack (dense and routed feed-forwards, a
+    layer reading an earlier layer's latent cache, bigram embedding) for
+    tests and smoke runs (random weights)."""
+    from .hybrid_config import munerax_model_config
+
+    def mixer(**kw):
+        m = {"heads": 3, "dim": 16, "rot_dim": 8, "vdim": 24, "kv_rank": 40,
+             "rot": {"base": 10000.0, "dims": 8}, "scale": 0.2}
+        m.update(kw)
+        return m
+    moe = {"kind": "moe", "expert": {"ff": 48},
+           "router": {"experts": 6, "top": 2, "scale": 1.5,
+                      "groups": {"count": 3, "keep": 2}},
+           "shared": {"ff": 80}}
+    layers = [
+        {"type": "latent_attention", "mixer": mixer(),
+         "mlp": {"kind": "dense", "ff": 224}},
+        {"type": "latent_attention", "mixer": mixer(kv_from=0), "mlp": moe},
+        {"type": "latent_attention", "mixer": mixer(heads=2), "mlp": moe},
+    ]
+    return munerax_model_config({
+        "architecture": "Munerax",
+        "embedding": {"scale": 4.0, "bigram": {
+            "buckets": 211, "mul_prev": 29, "mul_cur": 11}},
+        "layers": layers, "norm": {"eps": 1e-5}, "vocab": 512,
+        "width": 192, "max_positions": 1024}, name="tiny-munerax-test")
+
+
+register(_tiny_munerax())

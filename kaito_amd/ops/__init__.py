@@ -35,7 +35,9 @@ for _g, _names in {
     "mix": ("causal_conv_update "
             "qk_norm_cache_write window_attention window_attention_tiles "
             "post_norm_residual rms_norm_cast residual_add_norm "
-            "clamped_glu sigmoid_mul"),
+            "clamped_glu sigmoid_mul gelu_glu relu2"),
+    "latent": ("bigram_embed latent_rope_cache_write latent_attention "
+               "latent_expand"),
     "delta": "gated_delta_rule rglru_scan",
     "decay": "mlstm_scan ssd_scan",
 }.items():
@@ -606,9 +608,97 @@ def clamped_glu(gu, limit: float, alpha: float = 1.702):
 
 
 def sigmoid_mul(x, gate):
-    """x [T, N] * sigmoid(gate [T, N]) (gate's row stride free)."""
+    """x [T, N] * sigmoid(gate [T, Ng]) (gate's row stride free); with
+    Ng < N each gate column serves N/Ng consecutive columns of x (one
+    gate per head)."""
     if x.is_cuda:
         out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
         _K.sigmoid_mul(out, x, gate)
         return out
     return torch_ref.sigmoid_mul(x, gate)
+
+
+def gelu_glu(gu):
+    """[gate | up] rows [T, 2F] -> gelu_tanh(gate) * up [T, F]."""
+    if gu.is_cuda:
+        out = torch.empty(gu.size(0), gu.size(1) // 2, dtype=gu.dtype,
+                          device=gu.device)
+        _K.gelu_glu(out, gu)
+        return out
+    return torch_ref.gelu_glu(gu)
+
+
+def relu2(x):
+    """relu(x)^2, element-wise, rows [T, N] (row stride free)."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _K.relu2(out, x)
+        return out
+    return torch_ref.relu2(x)
+
+
+# ---- latent attention (kernel group "latent") -----------------------------
+
+def bigram_embed(ids, embed, scale: float, table, buckets: int,
+                 mul_prev: int, mul_cur: int, prev_state, cu_seqlens,
+                 state_slots, seq_starts, token_seq):
+    """f32 rows embed[ids]*scale (+ the hashed bigram row: (previous *
+    mul_prev + token * mul_cur) mod buckets, row `buckets` for a
+    sequence's first token). The token before a chunk's first row comes
+    from prev_state [slots] int64, which is advanced to the chunk's last
+    token. table None: token embedding only."""
+    if ids.is_cuda:
+        out = torch.empty(ids.size(0), embed.size(1), dtype=torch.float32,
+                          device=ids.device)
+        none = torch.empty(0, dtype=embed.dtype, device=ids.device)
+        _K.bigram_embed(out, ids, embed, scale,
+                        table if table is not None else none, buckets,
+                        mul_prev, mul_cur,
+                        prev_state if table is not None else
+                        torch.empty(0, dtype=torch.long, device=ids.device),
+                        cu_seqlens, state_slots, seq_starts, token_seq)
+        return out
+    return torch_ref.bigram_embed(ids, embed, scale, table, buckets,
+                                  mul_prev, mul_cur, prev_state, cu_seqlens,
+                                  state_slots, seq_starts)
+
+
+def latent_rope_cache_write(q, dkv, norm_w, eps: float, cache, slot_mapping,
+                            positions, inv_freq, dim: int):
+    """Rotation of the last 2R dims of every head of q [T, H, dim + 2R]
+    (R = len(inv_freq); i paired with i + R; angle = position *
+    inv_freq[i] in f32) and, with dkv [T, rank + 2R] given (row stride
+    free), the latent row: RMS norm of the first rank dims with the f32
+    weight norm_w, rotation of the last 2R, scatter into the paged latent
+    cache [blocks, block_size, rank + 2R] at slot_mapping (negative slots
+    skipped). Returns q rotated, contiguous."""
+    if q.is_cuda:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        own = dkv is not None
+        _K.latent_rope_cache_write(
+            out, q, dkv if own else torch.empty(0, 0, dtype=q.dtype,
+                                                device=q.device),
+            norm_w if own else _none(None, q), eps,
+            cache if own else torch.empty(0, dtype=q.dtype, device=q.device),
+            slot_mapping, positions, inv_freq, dim)
+        return out
+    return torch_ref.latent_rope_cache_write(q, dkv, norm_w, eps, cache,
+                                             slot_mapping, positions,
+                                             inv_freq, dim)
+
+
+def latent_attention(q, cache, block_tables, token_seq, positions,
+                     scale: float, rank: int, sinks=None):
+    """Causal attention of latent-space queries [T, H, rank + P] over the
+    paged latent cache [blocks, block_size, rank + P]: score = q . row *
+    scale over rows 0..position of the row's sequence, optional per-head
+    sinks in the denominator, output = weighted sum of the rows' first
+    `rank` dims, [T, H, rank]. One pass over the cache serves all heads."""
+    if q.is_cuda:
+        out = torch.empty(q.size(0), q.size(1), rank, dtype=q.dtype,
+                          device=q.device)
+        _K.latent_attention(out, q, cache, block_tables, token_seq,
+                            positions, scale, _none(sinks, q))
+        return out
+    return torch_ref.latent_attention(q, cache, block_tables, token_seq,
+                                      positions, scale, rank, sinks)

@@ -548,4 +548,107 @@ def clamped_glu(gu, limit: float, alpha: float):
 
 
 def sigmoid_mul(x, gate):
-    return (x.float() * torch.sigmoid(gate.float())).to(x.dtype)
+    """x [T, N] * sigmoid(gate [T, Ng]); with Ng < N each gate column
+    serves N/Ng consecutive columns of x."""
+    g = torch.sigmoid(gate.float())
+    if gate.size(-1) != x.size(-1):
+        g = g.repeat_interleave(x.size(-1) // gate.size(-1), -1)
+    return (x.float() * g).to(x.dtype)
+
+
+def gelu_glu(gu):
+    """gu [T, 2F] = [gate | up] -> gelu_tanh(gate) * up."""
+    F_ = gu.size(-1) // 2
+    g = torch.nn.functional.gelu(gu[..., :F_].float(), approximate="tanh")
+    return (g * gu[..., F_:].float()).to(gu.dtype)
+
+
+def relu2(x):
+    return torch.relu(x.float()).square().to(x.dtype)
+
+
+def bigram_embed(ids, embed, scale: float, table, buckets: int,
+                 mul_prev: int, mul_cur: int, prev_state, cu_seqlens,
+                 state_slots, seq_starts):
+    """x[t] = embed[ids[t]] * scale (+ table[row(t)]) as f32 rows. With a
+    table, row(t) = (previous * mul_prev + ids[t] * mul_cur) mod buckets,
+    the previous token being the row before t in its chunk or, for a
+    chunk's first row, prev_state[slot] (a chunk starting at position 0
+    takes row `buckets`). prev_state [slots] int64 is advanced to each
+    chunk's last token."""
+    x = embed[ids].float() * scale
+    if table is None:
+        return x
+    idl = ids.tolist()
+    rows = torch.zeros(len(idl), dtype=torch.long)
+    for c0, c1, slot, start in _chunks(cu_seqlens, state_slots, seq_starts):
+        prev = int(prev_state[slot]) if start > 0 else -1
+        for t in range(c0, c1):
+            rows[t] = buckets if prev < 0 else \
+                (prev * mul_prev + idl[t] * mul_cur) % buckets
+            prev = idl[t]
+        prev_state[slot] = prev
+    valid = torch.zeros(len(idl), 1)
+    for c0, c1, _, _ in _chunks(cu_seqlens, state_slots, seq_starts):
+        valid[c0:c1] = 1.0
+    return x + table[rows].float() * valid
+
+
+def latent_rope_cache_write(q, dkv, norm_w, eps: float, cache, slot_mapping,
+                            positions, inv_freq, dim: int):
+    """q [T, H, dim + 2R]: the last 2R dims of every head rotate (i paired
+    with i + R, angle = position * inv_freq[i], f32). dkv [T, rank + 2R]
+    (or None): the first rank dims are RMS-normed with norm_w, the last
+    2R rotated, and the row is scattered into cache [blocks, block_size,
+    rank + 2R] at slot_mapping (negative: skipped). Returns q rotated."""
+    R = inv_freq.numel()
+    ang = positions.float()[:, None] * inv_freq.float()[None, :]
+    c, s = torch.cos(ang), torch.sin(ang)
+
+    def rot(t, cc, ss):
+        a, b = t[..., :R], t[..., R:]
+        return torch.cat([a * cc - b * ss, b * cc + a * ss], -1)
+    qf = q.float()
+    qr = torch.cat([qf[..., :dim],
+                    rot(qf[..., dim:], c[:, None], s[:, None])], -1)
+    if dkv is not None:
+        rank = dkv.size(-1) - 2 * R
+        lat = dkv[:, :rank].float()
+        lat = lat * torch.rsqrt(lat.pow(2).mean(-1, keepdim=True) + eps) \
+            * norm_w.float()
+        row = torch.cat([lat, rot(dkv[:, rank:].float(), c, s)], -1)
+        flat = cache.view(-1, cache.size(-1))
+        for t, slot in enumerate(slot_mapping.tolist()):
+            if slot >= 0:
+                flat[slot] = row[t].to(cache.dtype)
+    return qr.to(q.dtype)
+
+
+def latent_attention(q, cache, block_tables, token_seq, positions,
+                     scale: float, rank: int, sinks=None):
+    """Causal attention in the latent space. q [T, H, rank + P] (the
+    unrotated query already folded through the key up-projection), cache
+    [blocks, block_size, rank + P]; row t belongs to chunk token_seq[t]
+    (its block-table row; negative: padding) at position positions[t] and
+    sees cached rows 0..position. score = q . row * scale; with `sinks`
+    [H] the softmax denominator also holds exp(sink_h). Returns the
+    weighted sum of the rows' first `rank` dims, [T, H, rank]."""
+    T, H, DT = q.shape
+    bs = cache.size(1)
+    flat = cache.view(-1, DT)
+    out = torch.zeros(T, H, rank)
+    pos_l, seq_l = positions.tolist(), token_seq.tolist()
+    for t in range(T):
+        if seq_l[t] < 0:
+            continue
+        js = torch.arange(pos_l[t] + 1)
+        rows = flat[block_tables[seq_l[t]].long()[js // bs] * bs + js % bs]
+        rows = rows.float()
+        s = q[t].float() @ rows.t() * scale              # [H, n]
+        if sinks is not None:
+            s = torch.cat([s, sinks.float()[:, None]], 1)
+            w = torch.softmax(s, -1)[:, :-1]
+        else:
+            w = torch.softmax(s, -1)
+        out[t] = w @ rows[:, :rank]
+    return out.to(q.dtype)
