@@ -562,8 +562,8 @@ class LatentAttention(nn.Module):
         lat, tables = ops.latent_gather(kv, meta.block_tables, meta.ctx_lens)
         k_s, v_s = ops.latent_expand(
             F.linear(lat[:, :s.kv_rank], self.w_uk),
-            F.linear(lat[:, :s.kv_rank], self.w_uv), lat, H, D, V, Dp, Vp,
-            kv.size(1))
+            F.linear(lat[:, :s.kv_rank], self.w_uv), lat, H, D, V, s.kv_rank,
+            Dp, Vp, kv.size(1))
         T = qr.size(0)
         if Dp != D + R:
             qp = qr.new_zeros(T, H, Dp)

@@ -702,3 +702,42 @@ def latent_attention(q, cache, block_tables, token_seq, positions,
         return out
     return torch_ref.latent_attention(q, cache, block_tables, token_seq,
                                       positions, scale, rank, sinks)
+
+
+def latent_gather(cache, block_tables, ctx_lens):
+    """Whole pages of the step's sequences out of the paged latent cache:
+    chunk b's first ceil(ctx_lens[b] / block_size) pages, in block-table
+    order. Returns (rows [pages * block_size, row], scratch block tables
+    [B, max pages] int32 numbering the gathered pages consecutively).
+    ctx_lens is a host list, so the shapes are known without a device
+    read; rows past a sequence's length are whatever the page holds and
+    stay behind the causal mask."""
+    bs, mb = cache.size(1), block_tables.size(1)
+    counts = [-(-int(n) // bs) for n in ctx_lens]
+    idx, tables, base = [], [], 0
+    width = max(max(counts), 1)
+    for b, n in enumerate(counts):
+        idx.extend(range(b * mb, b * mb + n))
+        tables.append(list(range(base, base + n)) + [0] * (width - n))
+        base += n
+    dev = cache.device
+    pages = block_tables.reshape(-1)[
+        torch.tensor(idx, dtype=torch.long, device=dev)].long()
+    rows = cache[pages].reshape(-1, cache.size(2))
+    return rows, torch.tensor(tables, dtype=torch.int32, device=dev)
+
+
+def latent_expand(kn, vv, lat, H: int, D: int, V: int, rank: int, Dp: int,
+                  Vp: int, block_size: int):
+    """Step-local paged K/V scratch from gathered latent rows (GPU): kn
+    [N, H*D] and vv [N, H*V] are the up-projected unrotated keys and
+    values of rows lat [N, rank + P]; head h's key is [kn_h | lat's last P
+    dims | zeros] of width Dp, its value [vv_h | zeros] of width Vp.
+    Returns k [N / block_size, H, block_size, Dp], v [..., Vp]."""
+    pages = lat.size(0) // block_size
+    k_s = torch.empty(pages, H, block_size, Dp, dtype=lat.dtype,
+                      device=lat.device)
+    v_s = torch.empty(pages, H, block_size, Vp, dtype=lat.dtype,
+                      device=lat.device)
+    _K.latent_expand(k_s, v_s, kn, vv, lat, H, D, V, rank)
+    return k_s, v_s

@@ -45,6 +45,8 @@ GROUPS: Dict[str, List[str]] = {
     "delta": ["delta_rule.hip", "rglru.hip"],
     # scalar-decay matrix recurrences: mLSTM, state-space duality
     "decay": ["decay_recurrence.hip"],
+    # latent attention over a paged low-rank cache, hashed bigram embedding
+    "latent": ["latent_attention.hip"],
 }
 
 
