@@ -441,6 +441,9 @@ def _munerax_layer(entry: dict, index: int, layers: list) -> LayerSpec:
             if int(other[k]) != int(mx[k]):
                 raise ValueError(f"layer {index}: {k} differs from layer "
                                  f"{src}, whose cache it reads")
+        if float(other["rot"]["base"]) != float(rot["base"]):
+            raise ValueError(f"layer {index}: rotation differs from layer "
+                             f"{src}, whose rotated keys it reads")
     glu, moe = _munerax_ff(entry.get("mlp"))
     return LayerSpec(kind, latent=LatentAttnSpec(
         heads=int(mx["heads"]), dim=int(mx["dim"]),

@@ -173,8 +173,7 @@ class MoEMLP(nn.Module):
         T, H = x.shape
         sorted_tok, gates, offsets = self._route(x)
         fused_shapes = (x.is_cuda and x.dtype == torch.bfloat16
-                        and H % 64 == 0 and self.ie_local % 64 == 0
-                        and self.gated)
+                        and H % 64 == 0 and self.ie_local % 64 == 0)
         # under hipGraph capture the fused kernels are mandatory (the
         # per-expert loop reads segment sizes on the host): deepseek k=6
         # crosses TK=4096 at decode bs>682 and measured 30.9k vs timeout

@@ -307,7 +307,8 @@ def moe_gate_silu(act: torch.Tensor, x: torch.Tensor,
     """Fused MoE stage 1 (GPU only): gather rows by sorted token ids,
     gate/up grouped GEMM per expert, activation epilogue into `act`
     (act_mode 0 = SwiGLU, 1 = gpt-oss clamped swiglu; optional
-    per-expert [E, 2*IE] bias)."""
+    per-expert [E, 2*IE] bias; 2 = ungated squared relu with weights
+    [E, IE, H])."""
     b = bias if bias is not None else         torch.empty(0, dtype=x.dtype, device=x.device)
     _K.moe_gate_silu(act, x, w_gate_up, sorted_ids, offsets,
                                   b, act_mode, e_base, n_local_experts)

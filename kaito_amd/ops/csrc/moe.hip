@@ -13,7 +13,9 @@
 //     reading two ints — no moe-align padding, no token dropping, no
 //     host sync;
 //   * kernel 1: act[s, :] = silu(x[tok] @ Wg[e]^T) * (x[tok] @ Wu[e]^T)
-//     with the A rows GATHERED through sorted_ids;
+//     with the A rows GATHERED through sorted_ids; ungated experts
+//     (act_mode 2, weights [E, IE, H]) skip the second product:
+//     act[s, :] = relu(x[tok] @ Wu[e]^T)^2;
 //   * kernel 2: out[tok, :] += gate_s * (act[s] @ Wd[e]^T), scattered
 //     with f32 atomics.
 //
@@ -109,12 +111,12 @@ KAITO_DEV float moe_act_f(int mode, float g, float u) {
 
 // act[s, n] = silu(x[tok_s] @ Wg[e]^T) * (x[tok_s] @ Wu[e]^T)
 // grid: (max_m_tiles, n_local_experts, IE/BN); block 256.
-template <int BN>
+template <int BN, bool GATED = true>
 __global__ __launch_bounds__(256, 3)
 void moe_gate_silu_kernel(
     short* __restrict__ act,             // [TK, IE] bf16
     const short* __restrict__ x,         // [T, H] bf16
-    const short* __restrict__ w,         // [E, 2*IE, H] bf16
+    const short* __restrict__ w,         // [E, 2*IE, H] bf16 (ungated: IE)
     const int* __restrict__ sorted_ids,  // [TK]
     const int* __restrict__ offsets,     // [E+1] (global expert ids)
     const short* __restrict__ bias,      // [E, 2*IE] bf16 or nullptr
@@ -138,14 +140,15 @@ void moe_gate_silu_kernel(
   // bench_moe_kernels.py) and the saved LDS buys 2x the resident blocks
   __shared__ short lds_a[BM * BK];
   __shared__ short lds_bg[BN * BK];
-  __shared__ short lds_bu[BN * BK];
+  __shared__ short lds_bu[GATED ? BN * BK : 8];
   __shared__ int s_rows[BM];
   for (int i = threadIdx.x; i < BM; i += 256)
     s_rows[i] = sorted_ids[m0 + min(i, m_rem - 1)];
   __syncthreads();
 
-  const short* wg = w + (int64_t)e * (2 * IE) * H + (int64_t)n0 * H;
-  const short* wu = wg + (int64_t)IE * H;
+  const short* wg = w + (int64_t)e * ((GATED ? 2 : 1) * IE) * H
+      + (int64_t)n0 * H;
+  const short* wu = wg + (int64_t)IE * H;   // gated only
 
   f32x4 accg[2][NR], accu[2][NR];
 #pragma unroll
@@ -159,7 +162,7 @@ void moe_gate_silu_kernel(
   for (int k0 = 0; k0 < H; k0 += BK) {
     stage_tile_gathered<BM>(x + k0, H, s_rows, lds_a, wave, lane);
     stage_tile_rows<BN>(wg + k0, H, lds_bg, wave, lane);
-    stage_tile_rows<BN>(wu + k0, H, lds_bu, wave, lane);
+    if constexpr (GATED) stage_tile_rows<BN>(wu + k0, H, lds_bu, wave, lane);
     __syncthreads();
 #pragma unroll
     for (int kk = 0; kk < BK / 32; kk++) {
@@ -170,7 +173,8 @@ void moe_gate_silu_kernel(
 #pragma unroll
       for (int b = 0; b < NR; b++) {
         bg[b] = frag_read(lds_bg, wn * (BN / 2) + b * 16 + lo, kk, hi);
-        bu[b] = frag_read(lds_bu, wn * (BN / 2) + b * 16 + lo, kk, hi);
+        if constexpr (GATED)
+          bu[b] = frag_read(lds_bu, wn * (BN / 2) + b * 16 + lo, kk, hi);
       }
 #pragma unroll
       for (int a = 0; a < 2; a++)
@@ -178,8 +182,9 @@ void moe_gate_silu_kernel(
         for (int b = 0; b < NR; b++) {
           accg[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
               af[a], bg[b], accg[a][b], 0, 0, 0);
-          accu[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              af[a], bu[b], accu[a][b], 0, 0, 0);
+          if constexpr (GATED)
+            accu[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                af[a], bu[b], accu[a][b], 0, 0, 0);
         }
     }
     __syncthreads();
@@ -198,6 +203,11 @@ void moe_gate_silu_kernel(
       for (int b = 0; b < NR; b++) {
         const int col = n0 + wn * (BN / 2) + b * 16 + lo;
         float g = accg[a][b][r], u = accu[a][b][r];
+        if constexpr (!GATED) {
+          const float m = fmaxf(g, 0.f);
+          act[(int64_t)(m0 + row) * IE + col] = f32_to_bf16(m * m);
+          continue;
+        }
         if (bias != nullptr) {
           g += bf16_to_f32(bias[(int64_t)e * 2 * IE + col]);
           u += bf16_to_f32(bias[(int64_t)e * 2 * IE + IE + col]);
@@ -309,7 +319,10 @@ void moe_gate_silu(at::Tensor act, at::Tensor x, at::Tensor w_gate_up,
   const int H = x.size(1);
   TORCH_CHECK(H % BK == 0 && IE % 64 == 0,
               "H/IE must be multiples of 64 for the fused MoE path");
-  TORCH_CHECK(w_gate_up.size(1) == 2 * IE && w_gate_up.size(2) == H);
+  const bool gated = act_mode != 2;
+  TORCH_CHECK(w_gate_up.size(1) == (gated ? 2 : 1) * IE &&
+              w_gate_up.size(2) == H);
+  TORCH_CHECK(gated || bias_ptr == nullptr, "ungated experts take no bias");
   const int mtiles = (TK + BM - 1) / BM;
   if (mtiles == 0 || n_local_experts == 0) return;
   auto stream = at::hip::getCurrentHIPStream();
@@ -317,6 +330,19 @@ void moe_gate_silu(at::Tensor act, at::Tensor x, at::Tensor w_gate_up,
   // n-tiles (the prefill-regime cost) at the same weight traffic
   const int BN = IE % 128 == 0 ? 128 : 64;
   dim3 grid(mtiles, n_local_experts, IE / BN), block(256);
+  if (!gated) {
+    if (BN == 128)
+      moe_gate_silu_kernel<128, false><<<grid, block, 0, stream>>>(
+          (short*)act.data_ptr(), (const short*)x.data_ptr(),
+          (const short*)w_gate_up.data_ptr(), sorted_ids.data_ptr<int>(),
+          offsets.data_ptr<int>(), nullptr, 2, (int)e_base, H, IE);
+    else
+      moe_gate_silu_kernel<64, false><<<grid, block, 0, stream>>>(
+          (short*)act.data_ptr(), (const short*)x.data_ptr(),
+          (const short*)w_gate_up.data_ptr(), sorted_ids.data_ptr<int>(),
+          offsets.data_ptr<int>(), nullptr, 2, (int)e_base, H, IE);
+    return;
+  }
   if (BN == 128)
     moe_gate_silu_kernel<128><<<grid, block, 0, stream>>>(
         (short*)act.data_ptr(), (const short*)x.data_ptr(),

@@ -577,21 +577,22 @@ def bigram_embed(ids, embed, scale: float, table, buckets: int,
     takes row `buckets`). prev_state [slots] int64 is advanced to each
     chunk's last token."""
     x = embed[ids].float() * scale
-    if table is None:
-        return x
     idl = ids.tolist()
+    valid = torch.zeros(len(idl), 1)
     rows = torch.zeros(len(idl), dtype=torch.long)
     for c0, c1, slot, start in _chunks(cu_seqlens, state_slots, seq_starts):
+        valid[c0:c1] = 1.0
+        if table is None:
+            continue
         prev = int(prev_state[slot]) if start > 0 else -1
         for t in range(c0, c1):
             rows[t] = buckets if prev < 0 else \
                 (prev * mul_prev + idl[t] * mul_cur) % buckets
             prev = idl[t]
         prev_state[slot] = prev
-    valid = torch.zeros(len(idl), 1)
-    for c0, c1, _, _ in _chunks(cu_seqlens, state_slots, seq_starts):
-        valid[c0:c1] = 1.0
-    return x + table[rows].float() * valid
+    if table is not None:
+        x = x + table[rows].float()
+    return x * valid          # rows of padding chunks are zero
 
 
 def latent_rope_cache_write(q, dkv, norm_w, eps: float, cache, slot_mapping,

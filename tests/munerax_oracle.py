@@ -101,9 +101,9 @@ def latent_attention(h, W, pre, mx, eps, kv):
     out = np.zeros((T, H, V))
     for i in range(T):
         for hh in range(H):
-            s = np.array([
-                (q_plain[i, hh] @ k_plain[j, hh] + q_rot[i, hh] @ kr[j])
-                * float(mx["scale"]) for j in range(i + 1)])
+            # keys 0..i: unrotated part per head, rotated part shared
+            s = (k_plain[:i + 1, hh] @ q_plain[i, hh]
+                 + kr[:i + 1] @ q_rot[i, hh]) * float(mx["scale"])
             m = max(s.max(), sink[hh])
             e = np.exp(s - m)
             den = e.sum() + math.exp(sink[hh] - m)
@@ -298,7 +298,15 @@ def write_checkpoint(folder, cfg, W):
     save_file({k: torch.from_numpy(np.asarray(v, dtype=np.float32)).to(
         torch.bfloat16).contiguous() for k, v in W.items()},
         os.path.join(folder, "model.safetensors"))
+    return folder
 
 
 def model_logits(cfg, W, tokens, streams=None):
-    return forward(cfg, W, list(tokens), streams)
+    """Logits [T, vocab] as a float64 torch tensor; `streams`, if a list,
+    receives the residual stream after every layer."""
+    import torch
+    raw = [] if streams is not None else None
+    out = torch.from_numpy(forward(cfg, W, list(tokens), raw))
+    if streams is not None:
+        streams.extend(torch.from_numpy(x) for x in raw)
+    return out
