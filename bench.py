@@ -60,7 +60,8 @@ def parse_args():
                         "random weights; comma-separated sizes of "
                         "kaito_amd.engine.hybrid_bench.SIZES (default all), "
                         "one JSON line per size and model; --hybrid-models "
-                        "picks from gurapel, pokulorn, swa-moe")
+                        "picks from gurapel, pokulorn, swa-moe, munerax, "
+                        "mla-moe (the latent-attention MoE transformer)")
     p.add_argument("--hybrid-batch", type=int, default=32)
     p.add_argument("--hybrid-prompt", type=int, default=2048)
     p.add_argument("--hybrid-out", type=int, default=128)

@@ -1,9 +1,10 @@
-"""Prefill and decode throughput of the hybrid stacks (Gurapel, Pokulorn)
-beside each other and beside the engine's closest homogeneous model at
-equal size: a sliding-window GQA transformer with the same MoE
-feed-forward (the gpt-oss class without sinks). Random weights, synthetic
-tokens; all models run through the same LLMEngine (scheduler, paged
-cache, hipGraph decode).
+"""Prefill and decode throughput of the hybrid stacks (Gurapel, Pokulorn,
+Munerax) beside each other and beside the engine's closest homogeneous
+model at equal size: a sliding-window GQA transformer with the same MoE
+feed-forward (the gpt-oss class without sinks) for the recurrent hybrids,
+the latent-attention MoE transformer (deepseek class) for Munerax. Random
+weights, synthetic tokens; all models run through the same LLMEngine
+(scheduler, paged cache, hipGraph decode).
 
 Used by `bench.py --hybrid-compare`; prints one JSON line per
 (size, model).
@@ -98,6 +99,65 @@ def transformer_config(name: str, z: dict, max_pos: int):
         sliding_window_pattern="all")
 
 
+# latent attention at the sizes of `z`: the head layout of the public
+# deepseek-v2-lite class (128 unrotated + 64 rotated key dims, 128 value
+# dims, latent rank 512), four expert groups of which two are eligible,
+# one shared expert as wide as a routed one
+LATENT = dict(dim=128, rot_dim=64, vdim=128, kv_rank=512, groups=4, keep=2,
+              scale=1.0)
+
+
+def munerax_config(name: str, z: dict, max_pos: int):
+    """The latent-attention stack: a dense first layer, then routed
+    layers, every third of which reads the latents of the layer before
+    it."""
+    from ..models.hybrid_config import munerax_model_config
+    a = LATENT
+    moe = {"kind": "moe", "expert": {"ff": z["ff"]},
+           "router": {"experts": z["experts"], "top": z["top"],
+                      "scale": a["scale"],
+                      "groups": {"count": a["groups"], "keep": a["keep"]}},
+           "shared": {"ff": z["ff"]}}
+
+    def layer(i):
+        mx = {"heads": z["heads"], "dim": a["dim"], "rot_dim": a["rot_dim"],
+              "vdim": a["vdim"], "kv_rank": a["kv_rank"],
+              "rot": {"base": 10000.0, "dims": a["rot_dim"]},
+              "scale": (a["dim"] + a["rot_dim"]) ** -0.5}
+        if i % 3 == 2:
+            mx["kv_from"] = i - 1
+        return {"type": "latent_attention", "mixer": mx,
+                "mlp": {"kind": "dense", "ff": z["ff"] * (z["top"] + 1)}
+                if i == 0 else moe}
+    return munerax_model_config({
+        "architecture": "Munerax",
+        "embedding": {"scale": 1.0, "bigram": {
+            "buckets": 65521, "mul_prev": 31, "mul_cur": 17}},
+        "layers": [layer(i) for i in range(z["layers"])],
+        "max_positions": max_pos, "norm": {"eps": 1e-5},
+        "vocab": z["vocab"], "width": z["width"]}, name=f"munerax-{name}")
+
+
+def latent_transformer_config(name: str, z: dict, max_pos: int):
+    """The engine's latent-attention MoE transformer (deepseek class) with
+    the same head layout, latent rank, experts, groups and shared
+    expert."""
+    from .config import ModelConfig
+    a = LATENT
+    return ModelConfig(
+        name=f"mla-moe-{name}", hidden_size=z["width"],
+        num_layers=z["layers"], num_heads=z["heads"],
+        num_kv_heads=z["heads"], head_dim=a["dim"] + a["rot_dim"],
+        intermediate_size=z["ff"] * (z["top"] + 1), vocab_size=z["vocab"],
+        max_position=max_pos, kv_lora_rank=a["kv_rank"], q_lora_rank=0,
+        qk_nope_head_dim=a["dim"], qk_rope_head_dim=a["rot_dim"],
+        v_head_dim=a["vdim"], num_experts=z["experts"],
+        num_experts_per_tok=z["top"], moe_intermediate_size=z["ff"],
+        moe_routing="noaux_tc", moe_norm_topk=False,
+        routed_scaling_factor=a["scale"], n_group=a["groups"],
+        topk_group=a["keep"], n_shared_experts=1, first_k_dense=1)
+
+
 def _measure(mcfg, batch: int, prompt: int, out_tokens: int, eager: bool):
     from .config import EngineConfig
     from .engine import LLMEngine
@@ -154,7 +214,10 @@ def run(sizes: List[str], batch: int, prompt: int, out_tokens: int,
         max_pos = prompt + out_tokens + 16
         for kind in models:
             mcfg = {"gurapel": hybrid_config, "pokulorn": pokulorn_config,
-                    "swa-moe": transformer_config}[kind](name, z, max_pos)
+                    "swa-moe": transformer_config,
+                    "munerax": munerax_config,
+                    "mla-moe": latent_transformer_config}[kind](
+                        name, z, max_pos)
             pre, dec = _measure(mcfg, batch, prompt, out_tokens, eager)
             row = {"bench": "hybrid-compare", "size": name, "model": kind,
                    "batch": batch, "prompt_tokens": prompt,

@@ -18,14 +18,18 @@
 //   latent_rope_cache_write   rotation of q's rotated part; RMS norm of the
 //                             latent + rotation of the shared key part +
 //                             scatter into the paged cache
-//   latent_attention          the latent-space attention above: workgroup
-//                             per (row, 8 heads), 32 cache rows per tile
+//   latent_attention          the latent-space attention above. bf16: MFMA
+//                             kernel, workgroup per (row, 16 heads, split
+//                             of the keys), partials joined by a merge
+//                             kernel. f32 and odd sizes: workgroup per
+//                             (row, 8 heads), 32 cache rows per tile
 //                             through LDS, online softmax, per-head sink
 //   latent_expand             packs up-projected keys/values of gathered
 //                             cache rows into a step-local paged K/V scratch
 //                             [pages, H, block_size, Dp|Vp] (zero padded)
 //                             for the MFMA prompt kernel of the window mixers
 #include "mix_common.h"
+#include <algorithm>
 
 namespace kaito {
 
@@ -231,6 +235,231 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
   }
 }
 
+// ---- latent-space attention on the matrix cores (bf16) -----------------------
+// Workgroup = one row x 16 heads x one split of the row's keys; 4 waves.
+// The 16 heads are the M side of v_mfma_f32_16x16x32_bf16. Per tile of 32
+// cache rows, staged once into LDS row-major (scores) and, for the first
+// `rank` dims, transposed (weighted sum):
+//   scores   S[16 x 32] = Q[16 x DT] K^T: the DT/32 k-steps are dealt to the
+//            4 waves (their query fragments stay in registers), partial sums
+//            meet in LDS;
+//   softmax  f32, thread (head, 2 keys), running maximum and sum per head in
+//            registers; weights leave as a bf16 value + remainder pair;
+//   sum      O[16 x rank] += P[16 x 32] C[32 x rank]: the rank/16 column
+//            tiles are dealt to the 4 waves, two MFMAs per tile (value and
+//            remainder), accumulators rescaled by the head's correction.
+// With S > 1 splits a workgroup covers a contiguous share of the key tiles
+// and leaves unnormalised (sum, maximum, denominator) partials for
+// latent_merge_kernel; the sink enters in split 0.
+constexpr int LM_KTP = 40;     // key stride of the transposed tile and of P
+
+template <int MAXKS, int NT>
+__global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
+    short* __restrict__ out,                        // [T, H, rank]
+    float* __restrict__ part_acc,                   // [T, S, H, rank]
+    float* __restrict__ part_ml,                    // [T, S, H, 2]
+    const short* __restrict__ q,                    // [T, H, DT]
+    const short* __restrict__ cache,                // [pages, BS, DT]
+    const int* __restrict__ block_tables, const int max_blocks,
+    const int* __restrict__ token_seq, const int64_t* __restrict__ positions,
+    const float scale, const float* __restrict__ sinks, const int H,
+    const int DT, const int rank, const int BS, const int S) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  const int DTp = (DT + 31) & ~31, RS = DTp + 8;
+  const int rankp = (rank + 15) & ~15;
+  short* kv_s = reinterpret_cast<short*>(lds_raw);          // [32][RS]
+  short* vt_s = kv_s + 32 * RS;                             // [rankp][KTP]
+  short* p_hi = vt_s + rankp * LM_KTP;                      // [16][KTP]
+  short* p_lo = p_hi + 16 * LM_KTP;                         // [16][KTP]
+  float* part_s = reinterpret_cast<float*>(p_lo + 16 * LM_KTP);  // [4][16][32]
+  float* s_corr = part_s + 4 * 16 * 32;                     // [16]
+  float* s_l = s_corr + 16;                                 // [16]
+  float* s_m = s_l + 16;                                    // [16]
+
+  const int t = blockIdx.x, h0 = blockIdx.y * 16, split = blockIdx.z;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int lo = lane & 15, hi = lane >> 4;
+  const int sh = tid >> 4, sj = tid & 15;       // softmax role: head, key pair
+  const int b = token_seq[t];
+  const int nkeys = b < 0 ? 0 : (int)positions[t] + 1;
+  const int nt_all = (nkeys + 31) >> 5;
+  const int tile_lo = (int)((int64_t)nt_all * split / S);
+  const int tile_hi = (int)((int64_t)nt_all * (split + 1) / S);
+  const int* bt = block_tables + (int64_t)max(b, 0) * max_blocks;
+
+  // zero what staging never writes: the k padding of the rows and the
+  // rows of the transposed tile past the rank
+  for (int i = tid; i < 32 * (RS - DT); i += 256)
+    kv_s[(i / (RS - DT)) * RS + DT + i % (RS - DT)] = 0;
+  for (int i = tid; i < (rankp - rank) * LM_KTP; i += 256)
+    vt_s[rank * LM_KTP + i] = 0;
+
+  // this wave's query fragments: k-steps wave, wave + 4, ...
+  const int nks = DTp >> 5;
+  bf16x8 qf[MAXKS];
+#pragma unroll
+  for (int i = 0; i < MAXKS; i++) {
+    const int d = ((wave + 4 * i) << 5) + hi * 8;
+    bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (h0 + lo < H && d < DT)
+      v = *reinterpret_cast<const bf16x8*>(
+          q + ((int64_t)t * H + h0 + lo) * DT + d);
+    qf[i] = v;
+  }
+  f32x4 acc[NT];
+#pragma unroll
+  for (int i = 0; i < NT; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bool sink = sinks != nullptr && split == 0 && h0 + sh < H;
+  float m_run = sink ? sinks[h0 + sh] : -INFINITY;
+  float l_run = sink ? 1.0f : 0.f;
+  const int nchunk = DT >> 3, key = tid & 31;
+
+  for (int tile = tile_lo; tile < tile_hi; tile++) {
+    const int k0 = tile << 5;
+    const int nk = min(32, nkeys - k0);
+    __syncthreads();            // previous tile consumed
+    {
+      const int j = k0 + key;
+      const short* src = key < nk
+          ? cache + ((int64_t)bt[j / BS] * BS + j % BS) * DT : nullptr;
+      for (int dc = tid >> 5; dc < nchunk; dc += 8) {
+        bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (src != nullptr) v = *reinterpret_cast<const bf16x8*>(src + dc * 8);
+        *reinterpret_cast<bf16x8*>(kv_s + key * RS + dc * 8) = v;
+        if (dc * 8 < rank) {
+#pragma unroll
+          for (int i = 0; i < 8; i++)
+            vt_s[(dc * 8 + i) * LM_KTP + key] = v[i];
+        }
+      }
+    }
+    __syncthreads();
+    // scores: partial over this wave's k-steps
+    f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+    for (int i = 0; i < MAXKS; i++) {
+      const int ks = wave + 4 * i;
+      if (ks < nks) {
+#pragma unroll
+        for (int nt = 0; nt < 2; nt++) {
+          const bf16x8 kb = *reinterpret_cast<const bf16x8*>(
+              kv_s + (nt * 16 + lo) * RS + (ks << 5) + hi * 8);
+          sc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[i], kb, sc[nt],
+                                                           0, 0, 0);
+        }
+      }
+    }
+#pragma unroll
+    for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+      for (int r = 0; r < 4; r++)
+        part_s[(wave * 16 + hi * 4 + r) * 32 + nt * 16 + lo] = sc[nt][r];
+    __syncthreads();
+    // softmax: head sh, keys sj and sj + 16
+    {
+      float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; w++) {
+        s0 += part_s[(w * 16 + sh) * 32 + sj];
+        s1 += part_s[(w * 16 + sh) * 32 + sj + 16];
+      }
+      s0 = sj < nk ? s0 * scale : -INFINITY;
+      s1 = sj + 16 < nk ? s1 * scale : -INFINITY;
+      const float m_new =
+          fmaxf(m_run, group_reduce_max<16>(fmaxf(s0, s1)));
+      const float p0 = sj < nk ? expf(s0 - m_new) : 0.f;
+      const float p1 = sj + 16 < nk ? expf(s1 - m_new) : 0.f;
+      const float ps = group_reduce_sum<16>(p0 + p1);
+      const float corr = expf(m_run - m_new);
+      l_run = l_run * corr + ps;
+      m_run = m_new;
+      const short h0b = f32_to_bf16(p0), h1b = f32_to_bf16(p1);
+      p_hi[sh * LM_KTP + sj] = h0b;
+      p_hi[sh * LM_KTP + sj + 16] = h1b;
+      p_lo[sh * LM_KTP + sj] = f32_to_bf16(p0 - bf16_to_f32(h0b));
+      p_lo[sh * LM_KTP + sj + 16] = f32_to_bf16(p1 - bf16_to_f32(h1b));
+      if (sj == 0) s_corr[sh] = corr;
+    }
+    __syncthreads();
+    // weighted sum over this wave's column tiles
+    {
+      const bf16x8 ah = *reinterpret_cast<const bf16x8*>(
+          p_hi + lo * LM_KTP + hi * 8);
+      const bf16x8 al = *reinterpret_cast<const bf16x8*>(
+          p_lo + lo * LM_KTP + hi * 8);
+      float cr[4];
+#pragma unroll
+      for (int r = 0; r < 4; r++) cr[r] = s_corr[hi * 4 + r];
+#pragma unroll
+      for (int i = 0; i < NT; i++) {
+        const int n = wave + 4 * i;
+        if (n * 16 < rankp) {
+          const bf16x8 vb = *reinterpret_cast<const bf16x8*>(
+              vt_s + (n * 16 + lo) * LM_KTP + hi * 8);
+          f32x4 a = acc[i];
+#pragma unroll
+          for (int r = 0; r < 4; r++) a[r] *= cr[r];
+          a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, vb, a, 0, 0, 0);
+          a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, vb, a, 0, 0, 0);
+          acc[i] = a;
+        }
+      }
+    }
+  }
+  if (b < 0 && split == 0) { m_run = 0.f; l_run = 1.0f; }   // padding row: zeros
+  __syncthreads();
+  if (sj == 0) { s_l[sh] = l_run; s_m[sh] = m_run; }
+  __syncthreads();
+  if (S > 1 && sj == 0 && h0 + sh < H) {
+    float* ml = part_ml + (((int64_t)t * S + split) * H + h0 + sh) * 2;
+    ml[0] = m_run;
+    ml[1] = l_run;
+  }
+#pragma unroll
+  for (int i = 0; i < NT; i++) {
+    const int d = (wave + 4 * i) * 16 + lo;
+    if (d >= rank) continue;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int hh = hi * 4 + r;
+      if (h0 + hh >= H) continue;
+      if (S > 1) {
+        part_acc[(((int64_t)t * S + split) * H + h0 + hh) * rank + d] =
+            acc[i][r];
+      } else {
+        out[((int64_t)t * H + h0 + hh) * rank + d] =
+            f32_to_bf16(acc[i][r] / s_l[hh]);
+      }
+    }
+  }
+}
+
+// grid (T, H), block 64: joins the S partials of a (row, head).
+__global__ void latent_merge_kernel(short* __restrict__ out,
+                                    const float* __restrict__ part_acc,
+                                    const float* __restrict__ part_ml,
+                                    const int H, const int rank,
+                                    const int S) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  float M = -INFINITY;
+  for (int s = 0; s < S; s++)
+    M = fmaxf(M, part_ml[(((int64_t)t * S + s) * H + h) * 2]);
+  float L = 0.f;
+  for (int s = 0; s < S; s++) {
+    const float* ml = part_ml + (((int64_t)t * S + s) * H + h) * 2;
+    L += ml[1] * expf(ml[0] - M);
+  }
+  const float inv = 1.0f / L;
+  for (int d = threadIdx.x; d < rank; d += blockDim.x) {
+    float a = 0.f;
+    for (int s = 0; s < S; s++) {
+      const float w = expf(part_ml[(((int64_t)t * S + s) * H + h) * 2] - M);
+      a += w * part_acc[(((int64_t)t * S + s) * H + h) * rank + d];
+    }
+    out[((int64_t)t * H + h) * rank + d] = f32_to_bf16(a * inv);
+  }
+}
+
 // ---- expansion into a step-local K/V scratch -------------------------------
 // grid (N rows, H), one wave. Row n of the gathered cache rows lands in
 // scratch page n / BS, slot n % BS.
@@ -371,16 +600,62 @@ void latent_attention(at::Tensor out, at::Tensor q, at::Tensor cache,
   TORCH_CHECK((int64_t)cache.size(0) * BS < (1ll << 31));
   if (T == 0) return;
   auto stream = at::hip::getCurrentHIPStream();
+  // bf16 with 16-byte chunks per row: the MFMA kernel
+  if (q.dtype() == at::kBFloat16 && DT % 8 == 0 && rank % 8 == 0 &&
+      DT <= 640 && rank <= 512) {
+    const int tiles_h = (H + 15) / 16;
+    // enough workgroups for the chip when rows x head tiles are few
+    int S = 512 / std::max(1, T * tiles_h);
+    S = std::max(1, std::min(S, 16));
+    const int DTp = (DT + 31) & ~31, rankp = (rank + 15) & ~15;
+    const size_t lds = (size_t)(32 * (DTp + 8) + rankp * LM_KTP +
+                                2 * 16 * LM_KTP) * 2 +
+        (size_t)(4 * 16 * 32 + 48) * 4;
+    at::Tensor pacc, pml;
+    if (S > 1) {
+      pacc = at::empty({T, S, H, rank}, q.options().dtype(at::kFloat));
+      pml = at::empty({T, S, H, 2}, q.options().dtype(at::kFloat));
+    }
+    const bool small = DT <= 256 && rank <= 128;
+    auto launch = [&](auto kern) {
+      static bool raised = false;
+      if (!raised) {
+        HIP_CHECK_KAITO(hipFuncSetAttribute(
+            reinterpret_cast<const void*>(kern),
+            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        raised = true;
+      }
+      hipLaunchKernelGGL(kern, dim3(T, tiles_h, S), dim3(256), lds, stream,
+          (short*)out.data_ptr(), S > 1 ? pacc.data_ptr<float>() : nullptr,
+          S > 1 ? pml.data_ptr<float>() : nullptr,
+          (const short*)q.data_ptr(), (const short*)cache.data_ptr(),
+          block_tables.data_ptr<int>(), (int)block_tables.size(1),
+          token_seq.data_ptr<int>(), positions.data_ptr<int64_t>(),
+          (float)scale, sk ? sinks.data_ptr<float>() : nullptr, H, DT, rank,
+          BS, S);
+    };
+    if (small) launch(&latent_attention_mfma_kernel<2, 2>);
+    else launch(&latent_attention_mfma_kernel<5, 8>);
+    if (S > 1)
+      hipLaunchKernelGGL(latent_merge_kernel, dim3(T, H), dim3(64), 0, stream,
+          (short*)out.data_ptr(), pacc.data_ptr<float>(),
+          pml.data_ptr<float>(), H, rank, S);
+    return;
+  }
   const int pad = q.dtype() == at::kFloat ? 1 : 2;
   const size_t lds = (size_t)(LA_HT * DT + LA_HT * LA_KT) * 4 +
       (size_t)LA_KT * (DT + pad) * q.element_size();
   TORCH_CHECK(lds <= 160 * 1024, "latent row too wide for this kernel: ", DT);
   TORCH_CHECK(H <= 65535 * LA_HT);
   KAITO_DISPATCH_ACT(q, {
-    if (lds > 48 * 1024)
+    // raised once per element type, to the most a workgroup may take
+    static bool raised = false;
+    if (lds > 48 * 1024 && !raised) {
       HIP_CHECK_KAITO(hipFuncSetAttribute(
           reinterpret_cast<const void*>(&latent_attention_kernel<act_t>),
-          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+      raised = true;
+    }
     hipLaunchKernelGGL((latent_attention_kernel<act_t>),
         dim3(T, (H + LA_HT - 1) / LA_HT), dim3(256), lds, stream,
         (act_t*)out.data_ptr(), (const act_t*)q.data_ptr(),

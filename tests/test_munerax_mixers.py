@@ -2,7 +2,9 @@
 package against the plain functions of tests/munerax_oracle.py or a
 closed form: hashed bigram embedding with its previous-token state,
 rotation + latent norm + paged cache write, latent-space attention (sink,
-far keys, page borders, more heads than a kernel tile, padding rows), the
+far keys, page borders, more heads than a kernel tile, padding rows; sizes
+for the simple and for the matrix-core kernel, which also splits the keys
+of a row over workgroups), the
 expanded prompt path against the latent path, group-limited sigmoid
 routing, squared-relu experts with a shared expert, and the element-wise
 gates. CPU runs check the reference ops; `-m gpu` runs the HIP kernels in
@@ -170,7 +172,8 @@ def paged(rows_per_seq, DT, dt, dev, pages=64, seed=0):
 
 
 @pytest.mark.parametrize("mode", MODES)
-@pytest.mark.parametrize("shape", [(3, 20, 4), (11, 33, 2), (16, 64, 16)])
+@pytest.mark.parametrize("shape", [(3, 20, 4), (11, 33, 2), (16, 64, 16),
+                                   (20, 160, 32)])
 def test_latent_attention_rows_of_mixed_steps(mode, shape):
     """Rows of several sequences at unequal positions (first tokens, page
     borders, mid-page) in one call, heads beyond one tile of 8, a padding
@@ -210,7 +213,7 @@ def test_far_key_found_among_hundreds(mode, far):
     so the output must be that key's latent: at the first position, at
     page borders, and at the query's own position."""
     dev, dt = mode
-    H, rank, P, n = 2, 12, 4, 300
+    H, rank, P, n = 2, 16, 8, 300
     DT = rank + P
     rng = np.random.default_rng(far)
     rows = M._bf16_round(rng.normal(0, 0.05, (n, DT)))
@@ -242,7 +245,7 @@ def test_sink_takes_its_share(mode):
     """With every score zero and n keys, the weights are 1 / (n + e^sink):
     the sink counts once, unscaled, and has no value."""
     dev, dt = mode
-    H, rank, P, n = 3, 8, 2, 5
+    H, rank, P, n = 3, 8, 8, 5
     rows = np.zeros((n, rank + P))
     rows[:, :rank] = 1.0
     rows[:, rank:] = 0.0
