@@ -434,29 +434,39 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
   }
 }
 
-// grid (T, H), block 64: joins the S partials of a (row, head).
+// grid (T, H), block 128: joins the S <= 16 partials of a (row, head); a
+// thread owns 4 adjacent output dims (rank is a multiple of 8).
 __global__ void latent_merge_kernel(short* __restrict__ out,
                                     const float* __restrict__ part_acc,
                                     const float* __restrict__ part_ml,
                                     const int H, const int rank,
                                     const int S) {
   const int t = blockIdx.x, h = blockIdx.y;
+  const float* ml = part_ml + ((int64_t)t * S * H + h) * 2;
+  const int64_t ml_step = (int64_t)H * 2, acc_step = (int64_t)H * rank;
+  float w[16];
   float M = -INFINITY;
-  for (int s = 0; s < S; s++)
-    M = fmaxf(M, part_ml[(((int64_t)t * S + s) * H + h) * 2]);
+#pragma unroll
+  for (int s = 0; s < 16; s++)
+    if (s < S) M = fmaxf(M, ml[s * ml_step]);
   float L = 0.f;
-  for (int s = 0; s < S; s++) {
-    const float* ml = part_ml + (((int64_t)t * S + s) * H + h) * 2;
-    L += ml[1] * expf(ml[0] - M);
+#pragma unroll
+  for (int s = 0; s < 16; s++) {
+    w[s] = s < S ? expf(ml[s * ml_step] - M) : 0.f;
+    if (s < S) L += ml[s * ml_step + 1] * w[s];
   }
   const float inv = 1.0f / L;
-  for (int d = threadIdx.x; d < rank; d += blockDim.x) {
-    float a = 0.f;
-    for (int s = 0; s < S; s++) {
-      const float w = expf(part_ml[(((int64_t)t * S + s) * H + h) * 2] - M);
-      a += w * part_acc[(((int64_t)t * S + s) * H + h) * rank + d];
-    }
-    out[((int64_t)t * H + h) * rank + d] = f32_to_bf16(a * inv);
+  const float* acc = part_acc + ((int64_t)t * S * H + h) * rank;
+  for (int d = threadIdx.x * 4; d < rank; d += blockDim.x * 4) {
+    float4_t a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 16; s++)
+      if (s < S)
+        a += w[s] * *reinterpret_cast<const float4_t*>(acc + s * acc_step + d);
+    short4_t o;
+#pragma unroll
+    for (int e = 0; e < 4; e++) o[e] = f32_to_bf16(a[e] * inv);
+    *reinterpret_cast<short4_t*>(out + ((int64_t)t * H + h) * rank + d) = o;
   }
 }
 
@@ -605,7 +615,8 @@ void latent_attention(at::Tensor out, at::Tensor q, at::Tensor cache,
       DT <= 640 && rank <= 512) {
     const int tiles_h = (H + 15) / 16;
     // enough workgroups for the chip when rows x head tiles are few
-    int S = 512 / std::max(1, T * tiles_h);
+    // (one workgroup per CU: a tile pair of 32 rows takes most of its LDS)
+    int S = (256 + T * tiles_h - 1) / std::max(1, T * tiles_h);
     S = std::max(1, std::min(S, 16));
     const int DTp = (DT + 31) & ~31, rankp = (rank + 15) & ~15;
     const size_t lds = (size_t)(32 * (DTp + 8) + rankp * LM_KTP +
@@ -637,7 +648,7 @@ void latent_attention(at::Tensor out, at::Tensor q, at::Tensor cache,
     if (small) launch(&latent_attention_mfma_kernel<2, 2>);
     else launch(&latent_attention_mfma_kernel<5, 8>);
     if (S > 1)
-      hipLaunchKernelGGL(latent_merge_kernel, dim3(T, H), dim3(64), 0, stream,
+      hipLaunchKernelGGL(latent_merge_kernel, dim3(T, H), dim3(128), 0, stream,
           (short*)out.data_ptr(), pacc.data_ptr<float>(),
           pml.data_ptr<float>(), H, rank, S);
     return;
