@@ -83,10 +83,11 @@ __global__ void bigram_state_kernel(int64_t* __restrict__ prev_state,
 }
 
 // ---- rotation + latent norm + cache scatter ----------------------------------
-// grid (T, H + 1), one wave. y < H: head y of q (first `dim` dims copied,
-// the 2R after them rotated). y == H: the latent row.
+// grid (T), 4 waves. The waves share the row's H + 1 items: item y < H is
+// head y of q (first `dim` dims copied, the 2R after them rotated), item H
+// the latent row (only for a mixer with a down-projection of its own).
 template <typename T>
-__global__ void latent_rope_cache_write_kernel(
+__global__ __launch_bounds__(256) void latent_rope_cache_write_kernel(
     T* __restrict__ q_out,                          // [T, H, dim + 2R]
     const T* __restrict__ q, const int64_t q_s0,    // [T, H, dim + 2R] view
     const T* __restrict__ dkv, const int64_t dkv_s0,   // [T, rank + 2R] view
@@ -95,38 +96,41 @@ __global__ void latent_rope_cache_write_kernel(
     const int64_t* __restrict__ positions,
     const float* __restrict__ inv_freq, const int H, const int dim,
     const int R, const int rank) {
-  const int t = blockIdx.x, y = blockIdx.y, lane = threadIdx.x;
+  const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float pos = (float)positions[t];
-  if (y < H) {
-    const int HD = dim + 2 * R;
-    const T* src = q + (int64_t)t * q_s0 + (int64_t)y * HD;
-    T* dst = q_out + ((int64_t)t * H + y) * HD;
-    for (int d = lane; d < dim; d += 64) dst[d] = src[d];
+  const int items = H + (dkv != nullptr ? 1 : 0);
+  const int HD = dim + 2 * R;
+  for (int y = wave; y < items; y += 4) {
+    if (y < H) {
+      const T* src = q + (int64_t)t * q_s0 + (int64_t)y * HD;
+      T* dst = q_out + ((int64_t)t * H + y) * HD;
+      for (int d = lane; d < dim; d += 64) dst[d] = src[d];
+      for (int i = lane; i < R; i += 64) {
+        const float ang = pos * inv_freq[i];
+        const float c = cosf(ang), s = sinf(ang);
+        const float u = act_ld(src + dim + i), v = act_ld(src + dim + R + i);
+        act_st(dst + dim + i, u * c - v * s);
+        act_st(dst + dim + R + i, v * c + u * s);
+      }
+      continue;
+    }
+    const int64_t slot = slot_mapping[t];
+    if (slot < 0) continue;
+    const T* src = dkv + (int64_t)t * dkv_s0;
+    T* dst = cache + slot * (int64_t)(rank + 2 * R);
+    float ss = 0.f;
+    for (int d = lane; d < rank; d += 64) { const float x = act_ld(src + d); ss += x * x; }
+    ss = wave_reduce_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)rank + eps);
+    for (int d = lane; d < rank; d += 64)
+      act_st(dst + d, act_ld(src + d) * inv * norm_w[d]);
     for (int i = lane; i < R; i += 64) {
       const float ang = pos * inv_freq[i];
       const float c = cosf(ang), s = sinf(ang);
-      const float u = act_ld(src + dim + i), v = act_ld(src + dim + R + i);
-      act_st(dst + dim + i, u * c - v * s);
-      act_st(dst + dim + R + i, v * c + u * s);
+      const float u = act_ld(src + rank + i), v = act_ld(src + rank + R + i);
+      act_st(dst + rank + i, u * c - v * s);
+      act_st(dst + rank + R + i, v * c + u * s);
     }
-    return;
-  }
-  const int64_t slot = slot_mapping[t];
-  if (slot < 0) return;
-  const T* src = dkv + (int64_t)t * dkv_s0;
-  T* dst = cache + slot * (int64_t)(rank + 2 * R);
-  float ss = 0.f;
-  for (int d = lane; d < rank; d += 64) { const float x = act_ld(src + d); ss += x * x; }
-  ss = wave_reduce_sum(ss);
-  const float inv = 1.0f / sqrtf(ss / (float)rank + eps);
-  for (int d = lane; d < rank; d += 64)
-    act_st(dst + d, act_ld(src + d) * inv * norm_w[d]);
-  for (int i = lane; i < R; i += 64) {
-    const float ang = pos * inv_freq[i];
-    const float c = cosf(ang), s = sinf(ang);
-    const float u = act_ld(src + rank + i), v = act_ld(src + rank + R + i);
-    act_st(dst + rank + i, u * c - v * s);
-    act_st(dst + rank + R + i, v * c + u * s);
   }
 }
 
@@ -573,10 +577,9 @@ void latent_rope_cache_write(at::Tensor q_out, at::Tensor q, at::Tensor dkv,
   }
   if (T == 0) return;
   auto stream = at::hip::getCurrentHIPStream();
-  TORCH_CHECK(H < 65535);
   KAITO_DISPATCH_ACT(q, {
     hipLaunchKernelGGL((latent_rope_cache_write_kernel<act_t>),
-        dim3(T, H + (own ? 1 : 0)), dim3(64), 0, stream,
+        dim3(T), dim3(256), 0, stream,
         (act_t*)q_out.data_ptr(), (const act_t*)q.data_ptr(), q.stride(0),
         own ? (const act_t*)dkv.data_ptr() : nullptr,
         own ? dkv.stride(0) : 0, own ? norm_w.data_ptr<float>() : nullptr,
