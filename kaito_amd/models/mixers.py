@@ -1,12 +1,11 @@
 """Token mixers for hybrid stacks: gated delta rule, real-gated linear
 recurrence, matrix-memory (mLSTM) recurrence, scalar-decay selective
-state space, and softmax attention over the paged cache in two flavours
+state space, softmax attention over the paged cache in two flavours
 (distance penalty without rotation; convolutions + rotation + window
 with kept first tokens + sink), and latent attention (one low-rank
 latent per token in the cache, optionally borrowed from an earlier
-layer). Each is a self-contained module
-parameterised by its spec (models/hybrid_config.py), so a design picks
-and combines them freely.
+layer). Each is a self-contained module parameterised by its spec
+(models/hybrid_config.py), so a design picks and combines them freely.
 
 All follow the same calling convention:
 
