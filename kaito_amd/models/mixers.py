@@ -531,10 +531,14 @@ class LatentAttention(nn.Module):
         q = p[:, :self.q_size].unflatten(-1, (H, D + s.rot_dim))
         dkv = p[:, self.q_size + self.g_size:] if self.own_kv else None
         kv = cache["kv"]
+        expanded = self._expanded_ok(x, meta)
+        # the MFMA prompt kernel takes key sizes 64/128/256: pad in place
+        pad = next(d for d in ops.WINDOW_MFMA_SIZES
+                   if d >= D + s.rot_dim) if expanded else 0
         qr = ops.latent_rope_cache_write(
             q, dkv, self.kv_norm, self.norm_eps, kv, meta.slot_mapping,
-            positions, self.inv_freq, D)
-        if self._expanded_ok(x, meta):
+            positions, self.inv_freq, D, pad_to=pad)
+        if expanded:
             o = self._expanded(qr, kv, meta)
         else:
             qc = torch.bmm(qr[..., :D].transpose(0, 1),
@@ -556,21 +560,15 @@ class LatentAttention(nn.Module):
         sequences in a step-local paged scratch, then the MFMA kernel."""
         s = self.spec
         H, D, R, V = s.heads, s.dim, s.rot_dim, s.vdim
-        Dp = next(d for d in ops.WINDOW_MFMA_SIZES if d >= D + R)
+        Dp = qr.size(2)                 # queries arrive zero-padded
         Vp = next(v for v in ops.WINDOW_MFMA_VSIZES if v >= V)
         lat, tables = ops.latent_gather(kv, meta.block_tables, meta.ctx_lens)
         k_s, v_s = ops.latent_expand(
             F.linear(lat[:, :s.kv_rank], self.w_uk),
             F.linear(lat[:, :s.kv_rank], self.w_uv), lat, H, D, V, s.kv_rank,
             Dp, Vp, kv.size(1))
-        T = qr.size(0)
-        if Dp != D + R:
-            qp = qr.new_zeros(T, H, Dp)
-            qp[..., :D + R] = qr
-        else:
-            qp = qr
         o = ops.window_attention(
-            qp, k_s, v_s, tables, meta.token_seq, None, s.scale,
+            qr, k_s, v_s, tables, meta.token_seq, None, s.scale,
             tiles=(meta.tile_seq, meta.tile_qbase, meta.cu_seqlens,
                    meta.seq_starts), sinks=self.sinks)
         return o[..., :V]

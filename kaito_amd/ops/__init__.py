@@ -665,16 +665,18 @@ def bigram_embed(ids, embed, scale: float, table, buckets: int,
 
 
 def latent_rope_cache_write(q, dkv, norm_w, eps: float, cache, slot_mapping,
-                            positions, inv_freq, dim: int):
+                            positions, inv_freq, dim: int, pad_to: int = 0):
     """Rotation of the last 2R dims of every head of q [T, H, dim + 2R]
     (R = len(inv_freq); i paired with i + R; angle = position *
     inv_freq[i] in f32) and, with dkv [T, rank + 2R] given (row stride
     free), the latent row: RMS norm of the first rank dims with the f32
     weight norm_w, rotation of the last 2R, scatter into the paged latent
     cache [blocks, block_size, rank + 2R] at slot_mapping (negative slots
-    skipped). Returns q rotated, contiguous."""
+    skipped). Returns q rotated, contiguous; with pad_to, every head is
+    zero-padded to that many dims."""
     if q.is_cuda:
-        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        out = torch.empty(q.size(0), q.size(1), max(pad_to, q.size(2)),
+                          dtype=q.dtype, device=q.device)
         own = dkv is not None
         _K.latent_rope_cache_write(
             out, q, dkv if own else torch.empty(0, 0, dtype=q.dtype,
@@ -683,9 +685,12 @@ def latent_rope_cache_write(q, dkv, norm_w, eps: float, cache, slot_mapping,
             cache if own else torch.empty(0, dtype=q.dtype, device=q.device),
             slot_mapping, positions, inv_freq, dim)
         return out
-    return torch_ref.latent_rope_cache_write(q, dkv, norm_w, eps, cache,
-                                             slot_mapping, positions,
-                                             inv_freq, dim)
+    out = torch_ref.latent_rope_cache_write(q, dkv, norm_w, eps, cache,
+                                            slot_mapping, positions,
+                                            inv_freq, dim)
+    if pad_to > out.size(2):
+        out = torch.nn.functional.pad(out, (0, pad_to - out.size(2)))
+    return out
 
 
 def latent_attention(q, cache, block_tables, token_seq, positions,

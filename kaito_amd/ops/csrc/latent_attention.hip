@@ -88,14 +88,14 @@ __global__ void bigram_state_kernel(int64_t* __restrict__ prev_state,
 // the latent row (only for a mixer with a down-projection of its own).
 template <typename T>
 __global__ __launch_bounds__(256) void latent_rope_cache_write_kernel(
-    T* __restrict__ q_out,                          // [T, H, dim + 2R]
+    T* __restrict__ q_out,                 // [T, H, HDo >= dim + 2R], 0-padded
     const T* __restrict__ q, const int64_t q_s0,    // [T, H, dim + 2R] view
     const T* __restrict__ dkv, const int64_t dkv_s0,   // [T, rank + 2R] view
     const float* __restrict__ norm_w, const float eps,
     T* __restrict__ cache, const int64_t* __restrict__ slot_mapping,
     const int64_t* __restrict__ positions,
     const float* __restrict__ inv_freq, const int H, const int dim,
-    const int R, const int rank) {
+    const int R, const int rank, const int HDo) {
   const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float pos = (float)positions[t];
   const int items = H + (dkv != nullptr ? 1 : 0);
@@ -103,8 +103,9 @@ __global__ __launch_bounds__(256) void latent_rope_cache_write_kernel(
   for (int y = wave; y < items; y += 4) {
     if (y < H) {
       const T* src = q + (int64_t)t * q_s0 + (int64_t)y * HD;
-      T* dst = q_out + ((int64_t)t * H + y) * HD;
+      T* dst = q_out + ((int64_t)t * H + y) * HDo;
       for (int d = lane; d < dim; d += 64) dst[d] = src[d];
+      for (int d = HD + lane; d < HDo; d += 64) act_st(dst + d, 0.f);
       for (int i = lane; i < R; i += 64) {
         const float ang = pos * inv_freq[i];
         const float c = cosf(ang), s = sinf(ang);
@@ -137,7 +138,7 @@ __global__ __launch_bounds__(256) void latent_rope_cache_write_kernel(
 // ---- latent-space attention ---------------------------------------------------
 constexpr int LA_HT = 8;      // heads per workgroup
 constexpr int LA_KT = 32;     // cache rows per tile
-constexpr int LA_MAXI = 16;   // rank <= 32 * LA_MAXI
+constexpr int LA_MAXI = 32;   // rank <= 32 * LA_MAXI
 
 template <typename T> struct lds_pad;                 // row padding, elements
 template <> struct lds_pad<float> { static constexpr int v = 1; };
@@ -558,7 +559,8 @@ void latent_rope_cache_write(at::Tensor q_out, at::Tensor q, at::Tensor dkv,
   TORCH_CHECK(R > 0 && dim >= 0 && dim + 2 * R == HD,
               "head size must be dim + 2 * len(inv_freq)");
   TORCH_CHECK(q_out.is_contiguous() && q_out.dtype() == q.dtype() &&
-              q_out.sizes() == q.sizes());
+              q_out.dim() == 3 && q_out.size(0) == T && q_out.size(1) == H &&
+              q_out.size(2) >= HD);
   TORCH_CHECK(positions.is_cuda() && positions.dtype() == at::kLong &&
               positions.is_contiguous() && positions.size(0) == T);
   const bool own = dkv.numel() > 0;
@@ -586,7 +588,7 @@ void latent_rope_cache_write(at::Tensor q_out, at::Tensor q, at::Tensor dkv,
         (float)eps, own ? (act_t*)cache.data_ptr() : nullptr,
         own ? slot_mapping.data_ptr<int64_t>() : nullptr,
         positions.data_ptr<int64_t>(), inv_freq.data_ptr<float>(), H,
-        (int)dim, R, rank);
+        (int)dim, R, rank, (int)q_out.size(2));
   });
 }
 

@@ -136,6 +136,14 @@ def test_rotation_norm_and_cache_write(mode):
         packed[:, :H * (D + R2)].unflatten(-1, (H, D + R2)), None, None, eps,
         cache, slots, torch.tensor(pos, dtype=torch.long, device=dev), inv, D)
     assert torch.equal(got_q, got_q2)
+    # zero-padded heads for a kernel that takes fixed key sizes
+    got_q3 = ops.latent_rope_cache_write(
+        packed[:, :H * (D + R2)].unflatten(-1, (H, D + R2)), None, None, eps,
+        cache, slots, torch.tensor(pos, dtype=torch.long, device=dev), inv, D,
+        pad_to=16)
+    assert got_q3.shape == (T, H, 16)
+    assert torch.equal(got_q3[..., :D + R2], got_q)
+    assert got_q3[..., D + R2:].abs().max().item() == 0.0
 
 
 # ---- latent-space attention ---------------------------------------------------------
