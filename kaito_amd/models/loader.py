@@ -454,7 +454,12 @@ def load_munerax_weights(model, path: str) -> None:
         put(layer.norm1, get(pre + "norm1").float())
         names = ("q",) + (("g",) if s.gate else ()) \
             + (("dkv",) if a.own_kv else ())
-        put(a.in_proj, torch.cat([get(ap + n) for n in names], 0))
+        w_in = torch.cat([get(ap + n) for n in names], 0)
+        if w_in.shape[0] != a.in_rows:
+            raise ValueError(f"{ap}: projection rows {w_in.shape[0]} vs "
+                             f"{a.in_rows} from the config")
+        put(a.in_proj, torch.nn.functional.pad(
+            w_in, (0, 0, 0, a.in_proj.shape[0] - a.in_rows)))
         if a.own_kv:
             put(a.kv_norm, get(ap + "dkv.norm").float())
         put(a.w_uk, get(ap + "uk"))

@@ -490,10 +490,12 @@ class LatentAttention(nn.Module):
         self.q_size = s.heads * (s.dim + s.rot_dim)
         self.g_size = s.heads if s.gate else 0
         self.row = s.kv_rank + s.rot_dim
-        # fused input projection, rows [q | gate | latent + rotated key]
-        self.in_proj = _p(self.q_size + self.g_size
-                          + (self.row if self.own_kv else 0), hidden,
-                          dtype=dtype)
+        # fused input projection, rows [q | gate | latent + rotated key],
+        # zero rows up to a multiple of 8 so that output rows stay 16-byte
+        # aligned for the kernels' vector moves
+        self.in_rows = self.q_size + self.g_size \
+            + (self.row if self.own_kv else 0)
+        self.in_proj = _p((self.in_rows + 7) // 8 * 8, hidden, dtype=dtype)
         self.kv_norm = _p(s.kv_rank, dtype=torch.float32) \
             if self.own_kv else None
         self.w_uk = _p(s.heads * s.dim, s.kv_rank, dtype=dtype)
@@ -529,7 +531,8 @@ class LatentAttention(nn.Module):
         T, H, D = x.size(0), s.heads, s.dim
         p = F.linear(x, self.in_proj)
         q = p[:, :self.q_size].unflatten(-1, (H, D + s.rot_dim))
-        dkv = p[:, self.q_size + self.g_size:] if self.own_kv else None
+        dkv = p[:, self.q_size + self.g_size:self.in_rows] \
+            if self.own_kv else None
         kv = cache["kv"]
         expanded = self._expanded_ok(x, meta)
         # the MFMA prompt kernel takes key sizes 64/128/256: pad in place

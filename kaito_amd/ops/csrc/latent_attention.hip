@@ -83,9 +83,10 @@ __global__ void bigram_state_kernel(int64_t* __restrict__ prev_state,
 }
 
 // ---- rotation + latent norm + cache scatter ----------------------------------
-// grid (T), 4 waves. The waves share the row's H + 1 items: item y < H is
-// head y of q (first `dim` dims copied, the 2R after them rotated), item H
-// the latent row (only for a mixer with a down-projection of its own).
+// grid (T, ceil(items / 4)), 4 waves, one item of the row per wave: item
+// y < H is head y of q (first `dim` dims copied, the 2R after them rotated,
+// the tail up to HDo zeroed; 16-byte moves when `vec`), item H the latent
+// row (only for a mixer with a down-projection of its own).
 template <typename T>
 __global__ __launch_bounds__(256) void latent_rope_cache_write_kernel(
     T* __restrict__ q_out,                 // [T, H, HDo >= dim + 2R], 0-padded
@@ -95,17 +96,29 @@ __global__ __launch_bounds__(256) void latent_rope_cache_write_kernel(
     T* __restrict__ cache, const int64_t* __restrict__ slot_mapping,
     const int64_t* __restrict__ positions,
     const float* __restrict__ inv_freq, const int H, const int dim,
-    const int R, const int rank, const int HDo) {
+    const int R, const int rank, const int HDo, const bool vec) {
   const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float pos = (float)positions[t];
   const int items = H + (dkv != nullptr ? 1 : 0);
   const int HD = dim + 2 * R;
-  for (int y = wave; y < items; y += 4) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  {
+    const int y = blockIdx.y * 4 + wave;
+    if (y >= items) return;
     if (y < H) {
       const T* src = q + (int64_t)t * q_s0 + (int64_t)y * HD;
       T* dst = q_out + ((int64_t)t * H + y) * HDo;
-      for (int d = lane; d < dim; d += 64) dst[d] = src[d];
-      for (int d = HD + lane; d < HDo; d += 64) act_st(dst + d, 0.f);
+      if (vec) {
+        for (int d = lane * VEC; d < dim; d += 64 * VEC)
+          *reinterpret_cast<float4_t*>(dst + d) =
+              *reinterpret_cast<const float4_t*>(src + d);
+        const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+        for (int d = HD + lane * VEC; d < HDo; d += 64 * VEC)
+          *reinterpret_cast<float4_t*>(dst + d) = zero;
+      } else {
+        for (int d = lane; d < dim; d += 64) dst[d] = src[d];
+        for (int d = HD + lane; d < HDo; d += 64) act_st(dst + d, 0.f);
+      }
       for (int i = lane; i < R; i += 64) {
         const float ang = pos * inv_freq[i];
         const float c = cosf(ang), s = sinf(ang);
@@ -113,10 +126,10 @@ __global__ __launch_bounds__(256) void latent_rope_cache_write_kernel(
         act_st(dst + dim + i, u * c - v * s);
         act_st(dst + dim + R + i, v * c + u * s);
       }
-      continue;
+      return;
     }
     const int64_t slot = slot_mapping[t];
-    if (slot < 0) continue;
+    if (slot < 0) return;
     const T* src = dkv + (int64_t)t * dkv_s0;
     T* dst = cache + slot * (int64_t)(rank + 2 * R);
     float ss = 0.f;
@@ -244,7 +257,8 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
 // Workgroup = one row x 16 heads x one split of the row's keys; 4 waves.
 // The 16 heads are the M side of v_mfma_f32_16x16x32_bf16. Per tile of 32
 // cache rows, staged once into LDS row-major (scores) and, for the first
-// `rank` dims, transposed (weighted sum):
+// `rank` dims, transposed (weighted sum), while the next tile's rows are
+// already being fetched into registers:
 //   scores   S[16 x 32] = Q[16 x DT] K^T: the DT/32 k-steps are dealt to the
 //            4 waves (their query fragments stay in registers), partial sums
 //            meet in LDS;
@@ -319,25 +333,54 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
   float l_run = sink ? 1.0f : 0.f;
   const int nchunk = DT >> 3, key = tid & 31;
 
+  // A thread owns cache row `key` of the tile and the 16-byte chunks
+  // tid/32, tid/32 + 8, ... of it. The next tile's chunks are fetched into
+  // registers while the current tile is computed.
+  constexpr int MAXC = 2 * MAXKS;
+  union chunk_t { bf16x8 v; uint32_t w[4]; };
+  chunk_t nxt[MAXC];
+  auto fetch = [&](const int tile) {
+    const int j = (tile << 5) + key;
+    const short* src = j < nkeys
+        ? cache + ((int64_t)bt[j / BS] * BS + j % BS) * DT : nullptr;
+#pragma unroll
+    for (int i = 0; i < MAXC; i++) {
+      const int dc = (tid >> 5) + 8 * i;
+      bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};     // rows past the end are zero
+      if (src != nullptr && dc < nchunk)
+        v = *reinterpret_cast<const bf16x8*>(src + dc * 8);
+      nxt[i].v = v;
+    }
+  };
+  if (tile_lo < tile_hi) fetch(tile_lo);
+  const bool odd = key & 1;
+
   for (int tile = tile_lo; tile < tile_hi; tile++) {
     const int k0 = tile << 5;
     const int nk = min(32, nkeys - k0);
     __syncthreads();            // previous tile consumed
-    {
-      const int j = k0 + key;
-      const short* src = key < nk
-          ? cache + ((int64_t)bt[j / BS] * BS + j % BS) * DT : nullptr;
-      for (int dc = tid >> 5; dc < nchunk; dc += 8) {
-        bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (src != nullptr) v = *reinterpret_cast<const bf16x8*>(src + dc * 8);
-        *reinterpret_cast<bf16x8*>(kv_s + key * RS + dc * 8) = v;
-        if (dc * 8 < rank) {
 #pragma unroll
-          for (int i = 0; i < 8; i++)
-            vt_s[(dc * 8 + i) * LM_KTP + key] = v[i];
+    for (int i = 0; i < MAXC; i++) {
+      const int dc = (tid >> 5) + 8 * i;
+      if (dc < nchunk) {
+        *reinterpret_cast<bf16x8*>(kv_s + key * RS + dc * 8) = nxt[i].v;
+        if (dc * 8 < rank) {
+          // transposed copy: neighbouring lanes hold neighbouring keys, so
+          // a pair trades halves and each lane stores two keys at once
+#pragma unroll
+          for (int jj = 0; jj < 4; jj++) {
+            const uint32_t own = nxt[i].w[jj];
+            const uint32_t oth = (uint32_t)__shfl_xor((int)own, 1, 64);
+            const uint32_t two = odd ? ((oth >> 16) | (own & 0xffff0000u))
+                                     : ((own & 0xffffu) | (oth << 16));
+            *reinterpret_cast<uint32_t*>(
+                vt_s + (dc * 8 + 2 * jj + (odd ? 1 : 0)) * LM_KTP +
+                (key & ~1)) = two;
+          }
         }
       }
     }
+    if (tile + 1 < tile_hi) fetch(tile + 1);
     __syncthreads();
     // scores: partial over this wave's k-steps
     f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
@@ -579,16 +622,24 @@ void latent_rope_cache_write(at::Tensor q_out, at::Tensor q, at::Tensor dkv,
   }
   if (T == 0) return;
   auto stream = at::hip::getCurrentHIPStream();
+  const int items = H + (own ? 1 : 0);
+  TORCH_CHECK(items <= 4 * 65535);
+  // 16-byte moves for the copied and the zeroed parts of a head
+  const int ve = 16 / (int)q.element_size();
+  const int HDo = q_out.size(2);
+  const bool vec = dim % ve == 0 && HD % ve == 0 && HDo % ve == 0 &&
+      q.stride(0) % ve == 0 && ((uintptr_t)q.data_ptr()) % 16 == 0 &&
+      ((uintptr_t)q_out.data_ptr()) % 16 == 0;
   KAITO_DISPATCH_ACT(q, {
     hipLaunchKernelGGL((latent_rope_cache_write_kernel<act_t>),
-        dim3(T), dim3(256), 0, stream,
+        dim3(T, (items + 3) / 4), dim3(256), 0, stream,
         (act_t*)q_out.data_ptr(), (const act_t*)q.data_ptr(), q.stride(0),
         own ? (const act_t*)dkv.data_ptr() : nullptr,
         own ? dkv.stride(0) : 0, own ? norm_w.data_ptr<float>() : nullptr,
         (float)eps, own ? (act_t*)cache.data_ptr() : nullptr,
         own ? slot_mapping.data_ptr<int64_t>() : nullptr,
         positions.data_ptr<int64_t>(), inv_freq.data_ptr<float>(), H,
-        (int)dim, R, rank, (int)q_out.size(2));
+        (int)dim, R, rank, HDo, vec);
   });
 }
 

@@ -91,10 +91,14 @@ def test_bigram_embedding_rows_and_state(mode):
 # ---- rotation, latent norm, cache write -----------------------------------------
 
 @pytest.mark.parametrize("mode", MODES)
-def test_rotation_norm_and_cache_write(mode):
+@pytest.mark.parametrize("sizes", [(3, 6, 4, 10, 3), (5, 16, 8, 24, 8)])
+def test_rotation_norm_and_cache_write(mode, sizes):
+    """Sizes with odd offsets (element-wise moves) and with 16-byte
+    aligned heads and rows (vector moves)."""
     dev, dt = mode
     rng = np.random.default_rng(1)
-    T, H, D, R2, rank, eps, base = 7, 3, 6, 4, 10, 1e-5, 50.0
+    H, D, R2, rank, gap = sizes
+    T, eps, base = 7, 1e-5, 50.0
     pos = [0, 1, 2, 40, 41, 500, 7]
     width = 12
     h = M._bf16_round(rng.normal(0, 1, (T, width)))
@@ -112,13 +116,13 @@ def test_rotation_norm_and_cache_write(mode):
     slots = torch.tensor([5, 16, 17, 31, 32, 639, -1], dtype=torch.long,
                          device=dev)
     # q and the latent row are column ranges of one projection output
-    packed = torch.zeros(T, H * (D + R2) + 3 + rank + R2, dtype=dt,
+    packed = torch.zeros(T, H * (D + R2) + gap + rank + R2, dtype=dt,
                          device=dev)
     packed[:, :H * (D + R2)] = torch.tensor(q.reshape(T, -1), dtype=dt)
-    packed[:, H * (D + R2) + 3:] = torch.tensor(d, dtype=dt)
+    packed[:, H * (D + R2) + gap:] = torch.tensor(d, dtype=dt)
     got_q = ops.latent_rope_cache_write(
         packed[:, :H * (D + R2)].unflatten(-1, (H, D + R2)),
-        packed[:, H * (D + R2) + 3:],
+        packed[:, H * (D + R2) + gap:],
         torch.tensor(W["m.dkv.norm"], dtype=torch.float32, device=dev), eps,
         cache, slots, torch.tensor(pos, dtype=torch.long, device=dev), inv, D)
     close(got_q, q_want, dt)
@@ -140,8 +144,8 @@ def test_rotation_norm_and_cache_write(mode):
     got_q3 = ops.latent_rope_cache_write(
         packed[:, :H * (D + R2)].unflatten(-1, (H, D + R2)), None, None, eps,
         cache, slots, torch.tensor(pos, dtype=torch.long, device=dev), inv, D,
-        pad_to=16)
-    assert got_q3.shape == (T, H, 16)
+        pad_to=32)
+    assert got_q3.shape == (T, H, 32)
     assert torch.equal(got_q3[..., :D + R2], got_q)
     assert got_q3[..., D + R2:].abs().max().item() == 0.0
 
@@ -286,7 +290,9 @@ def mixer_setup(dev, dt, H, D, R2, V, rank, width, seed, kv_from=None):
     with torch.no_grad():
         def t(name):
             return torch.tensor(W["l0.mix." + name])
-        m.in_proj.copy_(torch.cat([t("q"), t("g"), t("dkv")], 0).to(dt))
+        m.in_proj.zero_()
+        m.in_proj[:m.in_rows].copy_(
+            torch.cat([t("q"), t("g"), t("dkv")], 0).to(dt))
         m.kv_norm.copy_(t("dkv.norm").float())
         m.w_uk.copy_(t("uk").to(dt))
         m.w_uv.copy_(t("uv").to(dt))
