@@ -69,11 +69,16 @@ class ModelConfig:
     num_experts_per_tok: int = 2
     moe_intermediate_size: int = 0       # per-expert FFN width (0 → dense I)
     # expert activation: "silu" (SwiGLU) | "swiglu_oai" (gpt-oss clamped
-    # swiglu: (up+1) * gate*sigmoid(1.702*gate), clamp ±7)
+    # swiglu: (up+1) * gate*sigmoid(1.702*gate), clamp ±7) |
+    # "clamped_glu" (the same form with the clamp `moe_act_limit`) |
+    # "relu2" (ungated squared relu)
     moe_act: str = "silu"
+    moe_act_limit: float = 7.0
     moe_bias: bool = False               # per-expert gate_up/down biases
     # routing: "softmax_topk" (mixtral: softmax→topk→renorm) |
-    # "topk_softmax" (gpt-oss: topk logits→softmax over the k)
+    # "topk_softmax" (gpt-oss: topk logits→softmax over the k) |
+    # "softmax_bias" (softmax over all experts; the choice adds a
+    # per-expert correction, the weights are the plain scores)
     moe_routing: str = "softmax_topk"
     # router logits in f32 (x and the router matrix are widened before the
     # product) instead of the activation dtype
@@ -137,6 +142,9 @@ class ModelConfig:
     # hashed bigram table added to the token embedding
     # (models/hybrid_config.py BigramSpec); None = token embedding only
     bigram: Optional[object] = None
+    # a run of layers executed several times with the same weights
+    # (models/hybrid_config.py LoopSpec); None = every layer once
+    layer_loop: Optional[object] = None
 
     @classmethod
     def from_hf_config(cls, cfg: dict, name: str = "") -> "ModelConfig":

@@ -1,6 +1,6 @@
 """Per-layer specifications for hybrid stacks (recurrent, windowed and
 latent attention layers mixed in one model) and the config.json readers of
-the Gurapel, Pokulorn and Munerax designs.
+the Gurapel, Pokulorn, Munerax and Lokedra designs.
 
 A homogeneous model is described by the flat ModelConfig fields; a hybrid
 one additionally carries `layer_specs`, one LayerSpec per layer, each
@@ -64,9 +64,13 @@ class MoESpec:
     scores; experts form `groups` equal groups of neighbours, a group
     scores the sum of its two best experts, only the `keep_groups` best
     groups are eligible; weights are the chosen scores times `scale`, not
-    renormalised). `act`: "silu_glu" (gated experts) or "relu2" (ungated,
-    squared relu). `shared_ff` > 0 adds an always-on expert of that width
-    and the same form."""
+    renormalised) or "softmax_bias" (softmax over all experts; the choice
+    adds a per-expert correction to the scores, the weights are the chosen
+    scores without it, not renormalised). `act`: "silu_glu" (gated
+    experts), "relu2" (ungated, squared relu) or "clamped_glu"
+    (g = min(gate, limit), u = clamp(up, ±limit), g·sigmoid(1.702 g)·
+    (u + 1)). `shared_ff` > 0 adds an always-on expert of that width and
+    the same form."""
     experts: int
     top: int
     ff: int
@@ -76,12 +80,14 @@ class MoESpec:
     keep_groups: int = 1
     scale: float = 1.0
     shared_ff: int = 0
+    limit: float = 0.0            # clamp of "clamped_glu"
 
 
 @dataclass(frozen=True)
 class RotarySpec:
     """Rotation of the first `dims` dimensions of each q/k head, dimension
-    i paired with i + dims/2. With `factor` > 0 the frequencies are
+    i paired with i + dims/2, or with `interleaved` dimension 2i with
+    2i + 1. With `factor` > 0 the frequencies are
     interpolated by parts (wavelengths beyond `original`/`slow` turns are
     divided by `factor`, those below `original`/`fast` turns kept, a
     linear ramp between) and cos/sin are scaled by 0.1·ln(factor) + 1."""
@@ -91,6 +97,7 @@ class RotarySpec:
     original: float = 0.0
     fast: float = 32.0
     slow: float = 1.0
+    interleaved: bool = False
 
     def frequencies(self):
         """(per-pair angular frequencies as a float64 list, magnitude)."""
@@ -133,6 +140,12 @@ class RotaryAttnSpec:
     mix_values: bool = False
     gate: bool = False
     qk_norm: bool = True
+    # a chunked mask instead of a window: query i sees j <= i only with
+    # floor(i / chunk) == floor(j / chunk), chunks counted from position 0
+    chunk: int = 0
+    bias: bool = False            # biases on the q/k/v and output projections
+    tied_values: bool = False     # no value projection: v = k as cached
+    unit_sink: bool = False       # a sink of score 0: denominator 1 + sum
 
 
 @dataclass(frozen=True)
@@ -178,7 +191,8 @@ class LatentAttnSpec:
     and `vdim` value dimensions. Options: a per-head sink in the softmax
     denominator, a per-head sigmoid output gate, and `kv_from` = index of
     an earlier layer whose cached latent and rotated key this layer
-    reads instead of projecting its own."""
+    reads instead of projecting its own. `q_rank` > 0: queries are an
+    up-projection of an RMS-normed latent of that size."""
     heads: int
     dim: int
     rot_dim: int
@@ -189,6 +203,42 @@ class LatentAttnSpec:
     sink: bool = False
     gate: bool = False
     kv_from: Optional[int] = None
+    q_rank: int = 0
+
+
+@dataclass(frozen=True)
+class DiagDeltaSpec:
+    """Generalized delta rule: per head a [dim, dim] state with a decay per
+    key channel, removal along the unit key at a per-channel rate, and a
+    rank-one write: S <- diag(w) S - (a*u)(u^T S) + k v^T, u = k/|k|,
+    w = exp(-decay_rate * sigmoid(low-rank(h) + w0)), a = sigmoid(W_a h +
+    b). Read-out S^T r, unit RMS per head, a weight over all heads, a
+    sigmoid output gate."""
+    heads: int
+    dim: int
+    decay_rate: float = 0.6065306597126334     # exp(-1/2)
+    k_eps: float = 1e-6                         # inside the unit-key root
+
+
+@dataclass(frozen=True)
+class HGRN2Spec:
+    """Gated linear attention whose forget gate also sets what is written:
+    per head S <- diag(f) S + (1 - f) v^T, o = S^T q, q = silu(W_q h),
+    f = lower + (1 - lower) sigmoid(W_f h + b) per head and channel;
+    o is RMS-normed over vdim with a weight shared by the heads."""
+    heads: int
+    dim: int
+    vdim: int
+
+
+@dataclass(frozen=True)
+class LoopSpec:
+    """Layers start .. stop-1 run `times` times in a row with the same
+    weights (each pass with caches and states of its own); before every
+    pass but the first the embedding output is added to the stream."""
+    start: int
+    stop: int
+    times: int
 
 
 @dataclass(frozen=True)
@@ -216,6 +266,9 @@ class LayerSpec:
     # Pokulorn — "mlstm": MLSTMSpec; "attention": RotaryAttnSpec;
     # "parallel": RotaryAttnSpec beside SSDSpec, outputs summed with the
     # weights `branch_scales`.
+    # Lokedra — "general_delta": DiagDeltaSpec; "latent_attention":
+    # LatentAttnSpec; "parallel": RotaryAttnSpec beside HGRN2Spec, summed
+    # with `branch_scales`; feed-forward `moe` or none.
     kind: str
     delta: Optional[DeltaRuleSpec] = None
     attn: Optional[WindowAttnSpec] = None
@@ -228,6 +281,8 @@ class LayerSpec:
     branch_scales: Tuple[float, float] = (1.0, 1.0)
     latent: Optional[LatentAttnSpec] = None
     glu: Optional[GeluGLUSpec] = None
+    ddelta: Optional[DiagDeltaSpec] = None
+    hgrn: Optional[HGRN2Spec] = None
 
 
 def _moe_spec(m) -> Optional[MoESpec]:
@@ -312,7 +367,8 @@ def layer_moe_config(cfg: ModelConfig, moe: MoESpec) -> ModelConfig:
         moe_bias=False, n_shared_experts=0,
         moe_shared_intermediate_size=moe.shared_ff, n_group=moe.groups,
         topk_group=moe.keep_groups, moe_norm_topk=False,
-        routed_scaling_factor=moe.scale, moe_router_fp32=True)
+        routed_scaling_factor=moe.scale, moe_router_fp32=True,
+        moe_act_limit=moe.limit)
 
 
 # ---- Pokulorn ---------------------------------------------------------------
@@ -486,6 +542,95 @@ def munerax_model_config(cfg: dict, name: str = "",
                           mul_prev=int(bg["mul_prev"]),
                           mul_cur=int(bg["mul_cur"])) if bg else None,
         tie_word_embeddings=True, residual_fp32=True,
+        num_experts=moe.experts if moe else 0,
+        num_experts_per_tok=moe.top if moe else 0,
+        moe_intermediate_size=moe.ff if moe else 0, dtype=dtype)
+
+
+# ---- Lokedra ------------------------------------------------------------------
+
+def _lokedra_ff(m) -> Optional[MoESpec]:
+    if m is None:
+        return None
+    if m.get("kind", "moe") != "moe":
+        raise ValueError(f"unsupported feed-forward kind {m.get('kind')!r}")
+    return MoESpec(
+        experts=int(m["router"]["experts"]), top=int(m["router"]["top"]),
+        ff=int(m["expert"]["ff"]), routing="softmax_bias",
+        act="clamped_glu", limit=float(m["expert"]["limit"]))
+
+
+def _lokedra_layer(entry: dict) -> LayerSpec:
+    kind, mx = entry["type"], entry["mixer"]
+    moe = _lokedra_ff(entry.get("mlp"))
+    if kind == "general_delta":
+        return LayerSpec(kind, ddelta=DiagDeltaSpec(
+            heads=int(mx["heads"]), dim=int(mx["dim"])), moe=moe)
+    if kind == "latent_attention":
+        rot = _rotary_spec(mx["rot"])
+        if rot.dims != int(mx["rot_dim"]):
+            raise ValueError("the rotated key part is rotated whole")
+        return LayerSpec(kind, latent=LatentAttnSpec(
+            heads=int(mx["heads"]), dim=int(mx["dim"]),
+            rot_dim=int(mx["rot_dim"]), vdim=int(mx["vdim"]),
+            kv_rank=int(mx["kv_rank"]), scale=float(mx["scale"]),
+            rot=dataclasses.replace(rot, interleaved=True),
+            q_rank=int(mx["q_rank"])), moe=moe)
+    if kind == "parallel":
+        lf, rt = mx["left"], mx["right"]
+        if int(lf.get("vdim", lf["dim"])) != int(lf["dim"]):
+            raise ValueError("values are the keys: vdim must equal dim")
+        mask = lf.get("mask") or {}
+        return LayerSpec(
+            kind,
+            rattn=RotaryAttnSpec(
+                heads=int(lf["heads"]), kv_heads=int(lf["kv_heads"]),
+                dim=int(lf["dim"]), vdim=int(lf["dim"]),
+                scale=float(lf["scale"]), conv_taps=int(lf.get("conv", 0)),
+                chunk=int(mask.get("size", 0)), qk_norm=False, bias=True,
+                tied_values=True, unit_sink=True),
+            hgrn=HGRN2Spec(heads=int(rt["heads"]), dim=int(rt["dim"]),
+                           vdim=int(rt["vdim"])),
+            branch_scales=(float(mx["left_scale"]), float(mx["right_scale"])),
+            moe=moe)
+    raise ValueError(f"unknown layer type {kind!r}")
+
+
+def is_lokedra_config(cfg: dict) -> bool:
+    return cfg.get("architecture") == "Lokedra"
+
+
+def lokedra_model_config(cfg: dict, name: str = "",
+                         dtype: torch.dtype = torch.bfloat16) -> ModelConfig:
+    """config.json of a Lokedra checkpoint → ModelConfig (every size, the
+    layer order, the loop and every per-model constant come from the
+    file). The design has no position table, so its length limit is the
+    engine's."""
+    specs: Tuple[LayerSpec, ...] = tuple(
+        _lokedra_layer(e) for e in cfg["layers"])
+    n = len(specs)
+    lp = cfg.get("loop")
+    loop = None
+    if lp:
+        loop = LoopSpec(start=int(lp["start"]), stop=int(lp["stop"]),
+                        times=int(lp["times"]))
+        if not (0 <= loop.start <= loop.stop <= n and loop.times >= 1):
+            raise ValueError(f"loop {lp} does not fit {n} layers")
+    width = int(cfg["width"])
+    att = next((s.latent for s in specs if s.latent is not None), None)
+    moe = next((s.moe for s in specs if s.moe is not None), None)
+    return ModelConfig(
+        name=name or "lokedra", arch="lokedra", layer_specs=specs,
+        layer_loop=loop, hidden_size=width, num_layers=n,
+        num_heads=att.heads if att else 1, num_kv_heads=1,
+        head_dim=att.dim + att.rot_dim if att else width,
+        intermediate_size=moe.ff if moe else width,
+        vocab_size=int(cfg["vocab"]),
+        max_position=int(cfg.get("max_positions",
+                                 POKULORN_DEFAULT_MAX_POSITION)),
+        rms_eps=float(cfg["norm"]["eps"]),
+        embed_scale=float(cfg["embedding"].get("scale", 1.0)),
+        rms_norm_offset=True, tie_word_embeddings=True, residual_fp32=True,
         num_experts=moe.experts if moe else 0,
         num_experts_per_tok=moe.top if moe else 0,
         moe_intermediate_size=moe.ff if moe else 0, dtype=dtype)

@@ -30,6 +30,8 @@ def load_safetensors_weights(model, path: str,
         return load_pokulorn_weights(model, path)
     if getattr(model.cfg, "arch", "llama") == "munerax":
         return load_munerax_weights(model, path)
+    if getattr(model.cfg, "arch", "llama") == "lokedra":
+        return load_lokedra_weights(model, path)
     from safetensors.torch import safe_open
 
     cfg = model.cfg
@@ -489,4 +491,96 @@ def load_munerax_weights(model, path: str) -> None:
         if mlp.w_shared_gate_up is not None:
             put(mlp.w_shared_gate_up, get(fp + "shared.up"))
             put(mlp.w_shared_down, get(fp + "shared.down"))
+    ck.warn_unused()
+
+
+def load_lokedra_weights(model, path: str) -> None:
+    """Lokedra checkpoint (flat tensor names, `l<i>.` per layer, mixer
+    tensors under `.mix.`, feed-forward under `.mlp.`, linear weights
+    [out, in]) → LokedraForCausalLM. Fuses each mixer's input
+    projections, folds the one-plus norm weights and the branch weights
+    into the layer scales, sizes the decay bottleneck by the checkpoint's
+    tensors, stacks the experts (zero-filled up to the kernels' tile
+    width) and widens per-channel tensors to f32."""
+    ck = _FlatCheckpoint(path)
+    get, put = ck.get, ck.put
+    cat = torch.cat
+
+    def one_plus(name):
+        return get(name).float() + 1.0
+
+    put(model.embed_tokens.weight, get("embed"))
+    put(model.norm, one_plus("final.norm"))
+    for i, layer in enumerate(model.layers):
+        pre, mp = f"l{i}.", f"l{i}.mix."
+        spec = layer.spec
+        put(layer.norm1, one_plus(pre + "norm1"))
+        put(layer.shift, get(pre + "shift").float())
+        ls1 = get(pre + "ls1").float()
+        if spec.kind == "general_delta":
+            m = layer.mixer
+            put(layer.scale_mix, ls1)
+            put(m.in_proj, cat([get(mp + n) for n in "rkvg"], 0))
+            w1 = get(mp + "w1")
+            if w1.shape[0] != m.decay_rank:
+                m.set_decay_rank(int(w1.shape[0]))
+            put(m.gate_proj, cat([get(mp + "a"), w1], 0))
+            put(m.a_bias, get(mp + "a.b").float())
+            put(m.w2, get(mp + "w2").float())
+            put(m.w0, get(mp + "w0").float())
+            put(m.out_norm, get(mp + "norm").float())
+            put(m.o_proj, get(mp + "o"))
+        elif spec.kind == "latent_attention":
+            a = layer.mixer
+            put(layer.scale_mix, ls1)
+            w_in = cat([get(mp + "dq"), get(mp + "dkv")], 0)
+            if w_in.shape[0] != a.in_rows:
+                raise ValueError(f"{mp}: projection rows {w_in.shape[0]} vs "
+                                 f"{a.in_rows} from the config")
+            put(a.in_proj, torch.nn.functional.pad(
+                w_in, (0, 0, 0, a.in_proj.shape[0] - a.in_rows)))
+            put(a.q_norm, get(mp + "dq.norm").float())
+            put(a.w_uq, get(mp + "uq"))
+            put(a.kv_norm, get(mp + "dkv.norm").float())
+            put(a.w_uk, get(mp + "uk"))
+            put(a.w_uv, get(mp + "uv"))
+            put(a.o_proj, get(mp + "o"))
+        else:
+            a, r = layer.attn, layer.hgrn
+            lp, rp = mp + "left.", mp + "right."
+            left, right = spec.branch_scales
+            put(layer.scale_mix, ls1 * left)
+            put(layer.scale_mix2, ls1 * right)
+            put(a.qkv_proj, cat([get(lp + "q"), get(lp + "k")], 0))
+            put(a.qkv_bias, cat([get(lp + "q.b"), get(lp + "k.b")], 0))
+            if a.conv_weight is not None:
+                put(a.conv_weight, cat([get(lp + "q.conv"),
+                                        get(lp + "k.conv")], 0).float())
+            put(a.o_proj, get(lp + "o"))
+            put(a.o_bias, get(lp + "o.b"))
+            put(r.in_proj, cat([get(rp + "q"), get(rp + "v")], 0))
+            put(r.f_proj, get(rp + "f"))
+            put(r.f_bias, get(rp + "f.b").float())
+            put(r.lower, get(rp + "lower").float())
+            put(r.out_norm, get(rp + "norm").float())
+            put(r.o_proj, get(rp + "o"))
+        mlp = layer.mlp
+        if mlp is None:
+            continue
+        fp = pre + "mlp."
+        put(layer.scale_ff, get(pre + "ls2").float())
+        put(mlp.gate, get(fp + "router").float())
+        put(mlp.e_score_correction_bias, get(fp + "correction").float())
+        ie = mlp.ie_local
+        with torch.no_grad():
+            mlp.w_gate_up.zero_()
+            mlp.w_down.zero_()
+            for e in range(mlp.num_experts):
+                g, u, d = (get(f"{fp}e{e}.{n}") for n in ("gate", "up",
+                                                          "down"))
+                ff = g.shape[0]
+                dt = mlp.w_gate_up.dtype
+                mlp.w_gate_up[e, :ff].copy_(g.to(dt))
+                mlp.w_gate_up[e, ie:ie + ff].copy_(u.to(dt))
+                mlp.w_down[e, :, :ff].copy_(d.to(dt))
     ck.warn_unused()

@@ -2,9 +2,11 @@
 recurrence, matrix-memory (mLSTM) recurrence, scalar-decay selective
 state space, softmax attention over the paged cache in two flavours
 (distance penalty without rotation; convolutions + rotation + window
-with kept first tokens + sink), and latent attention (one low-rank
-latent per token in the cache, optionally borrowed from an earlier
-layer). Each is a self-contained module parameterised by its spec
+with kept first tokens or a chunked mask + sink, optionally with the
+keys as values), latent attention (one low-rank latent per token in the
+cache, optionally borrowed from an earlier layer, optionally with
+low-rank queries), the generalized delta rule with per-channel decay, and
+gated linear attention with a tied write gate (HGRN2). Each is a self-contained module parameterised by its spec
 (models/hybrid_config.py), so a design picks and combines them freely.
 
 All follow the same calling convention:
@@ -31,9 +33,10 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .. import ops
-from .hybrid_config import (DeltaRuleSpec, DenseFFSpec, GeluGLUSpec,
-                            LatentAttnSpec, MLSTMSpec, RGLRUSpec,
-                            RotaryAttnSpec, SSDSpec, WindowAttnSpec)
+from .hybrid_config import (DeltaRuleSpec, DenseFFSpec, DiagDeltaSpec,
+                            GeluGLUSpec, HGRN2Spec, LatentAttnSpec,
+                            MLSTMSpec, RGLRUSpec, RotaryAttnSpec, SSDSpec,
+                            WindowAttnSpec)
 
 
 def _p(*shape, dtype):
@@ -231,9 +234,13 @@ class RotaryWindowAttention(nn.Module):
     and k a per-head RMS norm and a rotation of their first `rot.dims`
     dimensions; the mask is causal, optionally a sliding window that
     also keeps the first `keep_first` tokens; a per-head sink may join
-    the softmax denominator; values may be blended with those of the
-    stack's first value-mixing layer before they are cached; the heads'
-    outputs may be gated by sigmoid of a fourth projection."""
+    the softmax denominator (learned, or fixed at score 0); the mask may
+    instead be chunked (a query sees the earlier keys of its own block of
+    `chunk` positions); values may be blended with those of the stack's
+    first value-mixing layer before they are cached, or be the keys
+    themselves as cached (no value projection, one cache tensor); the
+    projections may carry biases; the heads' outputs may be gated by
+    sigmoid of a fourth projection."""
 
     def __init__(self, hidden: int, spec: RotaryAttnSpec, dtype,
                  norm_eps: float):
@@ -243,12 +250,17 @@ class RotaryWindowAttention(nn.Module):
         s = spec
         self.q_size = s.heads * s.dim
         self.k_size = s.kv_heads * s.dim
-        self.v_size = s.kv_heads * s.vdim
+        if s.tied_values:
+            assert s.vdim == s.dim and not s.mix_values
+        self.v_size = 0 if s.tied_values else s.kv_heads * s.vdim
         self.o_size = s.heads * s.vdim
         self.conv_ch = self.q_size + self.k_size + self.v_size
         # fused input projection, rows [q | k | v | gate]
         self.qkv_proj = _p(self.conv_ch + (self.o_size if s.gate else 0),
                            hidden, dtype=dtype)
+        self.qkv_bias = _p(self.qkv_proj.shape[0], dtype=dtype) \
+            if s.bias else None
+        self.o_bias = _p(hidden, dtype=dtype) if s.bias else None
         self.conv_weight = _p(self.conv_ch, s.conv_taps, dtype=torch.float32) \
             if s.conv_taps > 0 else None
         if s.qk_norm:
@@ -263,7 +275,12 @@ class RotaryWindowAttention(nn.Module):
                 freq, dtype=torch.float64).float(), persistent=False)
         else:
             self.inv_freq, self.rot_mag = None, 1.0
-        self.sinks = _p(s.heads, dtype=torch.float32) if s.sink else None
+        if s.unit_sink:
+            assert not s.sink
+            self.register_buffer("sinks", torch.zeros(
+                s.heads, dtype=torch.float32), persistent=False)
+        else:
+            self.sinks = _p(s.heads, dtype=torch.float32) if s.sink else None
         # blend weight of the first value-mixing layer's values; the first
         # such layer of a stack never reads it
         self.v_lambda = 0.0
@@ -274,9 +291,10 @@ class RotaryWindowAttention(nn.Module):
         out = {
             "k": torch.zeros(num_blocks, s.kv_heads, block_size, s.dim,
                              dtype=self.dtype, device=device),
-            "v": torch.zeros(num_blocks, s.kv_heads, block_size, s.vdim,
-                             dtype=self.dtype, device=device),
         }
+        if not s.tied_values:
+            out["v"] = torch.zeros(num_blocks, s.kv_heads, block_size,
+                                   s.vdim, dtype=self.dtype, device=device)
         if s.conv_taps > 0:
             out["conv"] = torch.zeros(num_slots, max(s.conv_taps - 1, 1),
                                       self.conv_ch, dtype=self.dtype,
@@ -288,12 +306,13 @@ class RotaryWindowAttention(nn.Module):
         esz = torch.empty(0, dtype=self.dtype).element_size()
         slot = max(s.conv_taps - 1, 1) * self.conv_ch * esz \
             if s.conv_taps > 0 else 0
-        return s.kv_heads * block_size * (s.dim + s.vdim) * esz, slot
+        vdim = 0 if s.tied_values else s.vdim
+        return s.kv_heads * block_size * (s.dim + vdim) * esz, slot
 
     def forward(self, x, positions, cache, meta):
         s = self.spec
         T = x.size(0)
-        p = F.linear(x, self.qkv_proj)
+        p = F.linear(x, self.qkv_proj, self.qkv_bias)
         qkv = p[:, :self.conv_ch]
         if s.conv_taps > 0:
             qkv = ops.causal_conv_update(
@@ -302,8 +321,9 @@ class RotaryWindowAttention(nn.Module):
         q = qkv[:, :self.q_size].unflatten(-1, (s.heads, s.dim))
         k = qkv[:, self.q_size:self.q_size + self.k_size].unflatten(
             -1, (s.kv_heads, s.dim))
-        v = qkv[:, self.q_size + self.k_size:].unflatten(
-            -1, (s.kv_heads, s.vdim))
+        v = k if s.tied_values else qkv[:, self.q_size + self.k_size:] \
+            .unflatten(-1, (s.kv_heads, s.vdim))
+        v_cache = cache["k"] if s.tied_values else cache["v"]
         v_first, lam = None, 0.0
         if s.mix_values:
             shared = meta.layer_shared
@@ -313,21 +333,22 @@ class RotaryWindowAttention(nn.Module):
                 shared["v_first"] = v
         qn = ops.qk_norm_cache_write(
             q, k, v, self.q_norm, self.k_norm, self.norm_eps, cache["k"],
-            cache["v"], meta.slot_mapping, positions=positions,
+            v_cache, meta.slot_mapping, positions=positions,
             inv_freq=self.inv_freq, rot_mag=self.rot_mag, v_first=v_first,
             v_lambda=lam)
         tiles = None
         if meta.tile_seq is not None:
             tiles = (meta.tile_seq, meta.tile_qbase, meta.cu_seqlens,
                      meta.seq_starts)
-        o = ops.window_attention(qn, cache["k"], cache["v"],
+        o = ops.window_attention(qn, cache["k"], v_cache,
                                  meta.block_tables, meta.token_seq, positions,
                                  s.scale, window=s.window, tiles=tiles,
-                                 keep_first=s.keep_first, sinks=self.sinks)
+                                 keep_first=s.keep_first, sinks=self.sinks,
+                                 chunk=s.chunk)
         o = o.reshape(T, self.o_size)
         if s.gate:
             o = ops.sigmoid_mul(o, p[:, self.conv_ch:])
-        return F.linear(o, self.o_proj)
+        return F.linear(o, self.o_proj, self.o_bias)
 
 
 class MLSTMMixer(nn.Module):
@@ -464,8 +485,10 @@ class LatentAttention(nn.Module):
     `rot_dim` dims shared by all heads; head h's key is [W_uk,h c | rotated
     part] and its value W_uv,h c. Queries carry `dim` unrotated and
     `rot_dim` rotated dims per head. Options: per-head sink in the softmax
-    denominator, per-head sigmoid output gate read from the mixer input.
-    With spec.kv_from set the mixer has no down-projection and reads the
+    denominator, per-head sigmoid output gate read from the mixer input,
+    queries through an RMS-normed latent of their own (spec.q_rank), the
+    rotation pairing neighbours (2i, 2i + 1) and carrying interpolated
+    frequencies with a magnitude. With spec.kv_from set the mixer has no down-projection and reads the
     cache of the layer it names (the caller passes that layer's cache).
 
     Two equivalent evaluations (key and value are linear in c):
@@ -490,17 +513,21 @@ class LatentAttention(nn.Module):
         self.q_size = s.heads * (s.dim + s.rot_dim)
         self.g_size = s.heads if s.gate else 0
         self.row = s.kv_rank + s.rot_dim
-        # fused input projection, rows [q | gate | latent + rotated key],
-        # zero rows up to a multiple of 8 so that output rows stay 16-byte
-        # aligned for the kernels' vector moves
-        self.in_rows = self.q_size + self.g_size \
+        # fused input projection, rows [q (or its latent) | gate | latent +
+        # rotated key], zero rows up to a multiple of 8 so that output
+        # rows stay 16-byte aligned for the kernels' vector moves
+        self.q_rows = s.q_rank if s.q_rank > 0 else self.q_size
+        self.in_rows = self.q_rows + self.g_size \
             + (self.row if self.own_kv else 0)
+        if s.q_rank > 0:
+            self.q_norm = _p(s.q_rank, dtype=torch.float32)
+            self.w_uq = _p(self.q_size, s.q_rank, dtype=dtype)
         self.in_proj = _p((self.in_rows + 7) // 8 * 8, hidden, dtype=dtype)
         self.kv_norm = _p(s.kv_rank, dtype=torch.float32) \
             if self.own_kv else None
         self.w_uk = _p(s.heads * s.dim, s.kv_rank, dtype=dtype)
         self.w_uv = _p(s.heads * s.vdim, s.kv_rank, dtype=dtype)
-        freq, _ = s.rot.frequencies()
+        freq, self.rot_mag = s.rot.frequencies()
         self.register_buffer("inv_freq", torch.tensor(
             freq, dtype=torch.float64).float(), persistent=False)
         self.sinks = _p(s.heads, dtype=torch.float32) if s.sink else None
@@ -530,8 +557,13 @@ class LatentAttention(nn.Module):
         s = self.spec
         T, H, D = x.size(0), s.heads, s.dim
         p = F.linear(x, self.in_proj)
-        q = p[:, :self.q_size].unflatten(-1, (H, D + s.rot_dim))
-        dkv = p[:, self.q_size + self.g_size:self.in_rows] \
+        if s.q_rank > 0:
+            cq = ops.rms_norm_cast(p[:, :s.q_rank].contiguous(), self.q_norm,
+                                   self.norm_eps, self.dtype)
+            q = F.linear(cq, self.w_uq).unflatten(-1, (H, D + s.rot_dim))
+        else:
+            q = p[:, :self.q_size].unflatten(-1, (H, D + s.rot_dim))
+        dkv = p[:, self.q_rows + self.g_size:self.in_rows] \
             if self.own_kv else None
         kv = cache["kv"]
         expanded = self._expanded_ok(x, meta)
@@ -540,7 +572,8 @@ class LatentAttention(nn.Module):
                    if d >= D + s.rot_dim) if expanded else 0
         qr = ops.latent_rope_cache_write(
             q, dkv, self.kv_norm, self.norm_eps, kv, meta.slot_mapping,
-            positions, self.inv_freq, D, pad_to=pad)
+            positions, self.inv_freq, D, pad_to=pad,
+            interleaved=s.rot.interleaved, rot_mag=self.rot_mag)
         if expanded:
             o = self._expanded(qr, kv, meta)
         else:
@@ -555,7 +588,7 @@ class LatentAttention(nn.Module):
                           .transpose(1, 2)).transpose(0, 1)
         o = o.reshape(T, H * s.vdim)
         if s.gate:
-            o = ops.sigmoid_mul(o, p[:, self.q_size:self.q_size + H])
+            o = ops.sigmoid_mul(o, p[:, self.q_rows:self.q_rows + H])
         return F.linear(o, self.o_proj)
 
     def _expanded(self, qr, kv, meta):
@@ -588,3 +621,109 @@ class GeluGLU(nn.Module):
 
     def forward(self, x):
         return F.linear(ops.gelu_glu(F.linear(x, self.gate_up)), self.down)
+
+
+class DiagDeltaMixer(nn.Module):
+    """Generalized delta rule. Per head the state S is a [dim, dim] f32
+    matrix; per token, with the unit key u = k/|k|,
+        S <- diag(w) S - (a*u)(u^T S) + k v^T,      o = S^T r,
+    where the decay w = exp(-rate*sigmoid(W2 tanh(W1 x) + w0)) and the
+    removal rate a = sigmoid(W_a x + b) are per head and key channel. o is
+    divided by its RMS per head, weighted over all heads, gated by
+    sigmoid(W_g x) and projected out. r, k, v and the gate come from one
+    activation-dtype projection; the pre-activations of w and a from a
+    projection whose result stays f32 (they enter the recurrence)."""
+
+    def __init__(self, hidden: int, spec: DiagDeltaSpec, dtype,
+                 norm_eps: float, decay_rank: int = 32):
+        super().__init__()
+        self.spec, self.dtype, self.norm_eps = spec, dtype, norm_eps
+        self.hidden = hidden
+        self.n = spec.heads * spec.dim
+        # fused input projection, rows [r | k | v | gate]
+        self.in_proj = _p(4 * self.n, hidden, dtype=dtype)
+        self.a_bias = _p(self.n, dtype=torch.float32)
+        self.w0 = _p(self.n, dtype=torch.float32)
+        self.out_norm = _p(self.n, dtype=torch.float32)
+        self.o_proj = _p(hidden, self.n, dtype=dtype)
+        self.set_decay_rank(decay_rank)
+
+    def set_decay_rank(self, rank: int):
+        """(Re)create the low-rank decay path for a bottleneck of `rank`
+        (a checkpoint's tensor shapes decide it)."""
+        dev = self.in_proj.device
+        self.decay_rank = rank
+        # rows [removal rate a | decay bottleneck W1], f32 result
+        self.gate_proj = nn.Parameter(torch.empty(
+            self.n + rank, self.hidden, dtype=self.dtype, device=dev),
+            requires_grad=False)
+        self.w2 = nn.Parameter(torch.empty(
+            self.n, rank, dtype=torch.float32, device=dev),
+            requires_grad=False)
+
+    def alloc_cache(self, num_blocks, block_size, num_slots, device) -> Dict:
+        s = self.spec
+        return {"ssm": torch.zeros(num_slots, s.heads, s.dim, s.dim,
+                                   dtype=torch.float32, device=device)}
+
+    def cache_bytes(self, block_size: int):
+        s = self.spec
+        return 0, s.heads * s.dim * s.dim * 4
+
+    def forward(self, x, positions, cache, meta):
+        s = self.spec
+        n = self.n
+        p = F.linear(x, self.in_proj)
+        gp = ops.linear_f32(x, self.gate_proj)               # [T, n + rank]
+        w_pre = F.linear(torch.tanh(gp[:, n:]), self.w2, self.w0)
+        a_pre = gp[:, :n] + self.a_bias
+        hd = (s.heads, s.dim)
+        o = ops.diag_delta_rule(
+            p[:, :n].unflatten(-1, hd), p[:, n:2 * n].unflatten(-1, hd),
+            p[:, 2 * n:3 * n].unflatten(-1, hd), w_pre, a_pre,
+            p[:, 3 * n:].unflatten(-1, hd), self.out_norm, cache["ssm"],
+            meta.cu_seqlens, meta.state_slots, meta.seq_starts,
+            s.decay_rate, s.k_eps, self.norm_eps)
+        return F.linear(o, self.o_proj)
+
+
+class HGRN2Mixer(nn.Module):
+    """Gated linear attention in which the forget gate also decides what
+    is written: per head S <- diag(f) S + (1 - f) v^T, o = S^T q with
+    q = silu(W_q x) and f = lower + (1 - lower) sigmoid(W_f x + b) per head
+    and channel (f acts on the state rows that belong to q's channels).
+    o is RMS-normed over vdim with a weight shared by the heads and
+    projected out. The gate pre-activation stays f32."""
+
+    def __init__(self, hidden: int, spec: HGRN2Spec, dtype, norm_eps: float):
+        super().__init__()
+        self.spec, self.dtype, self.norm_eps = spec, dtype, norm_eps
+        s = spec
+        self.n_q = s.heads * s.dim
+        self.n_v = s.heads * s.vdim
+        self.in_proj = _p(self.n_q + self.n_v, hidden, dtype=dtype)  # [q | v]
+        self.f_proj = _p(self.n_q, hidden, dtype=dtype)
+        self.f_bias = _p(self.n_q, dtype=torch.float32)
+        self.lower = _p(self.n_q, dtype=torch.float32)
+        self.out_norm = _p(s.vdim, dtype=torch.float32)
+        self.o_proj = _p(hidden, self.n_v, dtype=dtype)
+
+    def alloc_cache(self, num_blocks, block_size, num_slots, device) -> Dict:
+        s = self.spec
+        return {"ssm": torch.zeros(num_slots, s.heads, s.dim, s.vdim,
+                                   dtype=torch.float32, device=device)}
+
+    def cache_bytes(self, block_size: int):
+        s = self.spec
+        return 0, s.heads * s.dim * s.vdim * 4
+
+    def forward(self, x, positions, cache, meta):
+        s = self.spec
+        p = F.linear(x, self.in_proj)
+        f_pre = ops.linear_f32(x, self.f_proj, self.f_bias)
+        o = ops.hgrn2_scan(
+            p[:, :self.n_q].unflatten(-1, (s.heads, s.dim)),
+            p[:, self.n_q:].unflatten(-1, (s.heads, s.vdim)), f_pre,
+            self.lower, self.out_norm, cache["ssm"], meta.cu_seqlens,
+            meta.state_slots, meta.seq_starts, self.norm_eps)
+        return F.linear(o, self.o_proj)

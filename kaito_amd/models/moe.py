@@ -80,9 +80,12 @@ class MoEMLP(nn.Module):
         else:
             self.b_gate_up = None
             self.b_down = None
-        self.act_mode = {"swiglu_oai": 1, "relu2": 2}.get(cfg.moe_act, 0)
-        # deepseek-v3 noaux_tc routing: per-expert selection bias
-        if cfg.moe_routing == "noaux_tc":
+        self.act_mode = {"swiglu_oai": 1, "clamped_glu": 1,
+                         "relu2": 2}.get(cfg.moe_act, 0)
+        self.act_limit = float(cfg.moe_act_limit) \
+            if cfg.moe_act == "clamped_glu" else 7.0
+        # per-expert selection bias (deepseek-v3 noaux_tc; softmax_bias)
+        if cfg.moe_routing in ("noaux_tc", "softmax_bias"):
             self.e_score_correction_bias = nn.Parameter(
                 torch.empty(e, dtype=torch.float32), requires_grad=False)
         # deepseek shared experts: always-on dense SwiGLU of width
@@ -133,6 +136,13 @@ class MoEMLP(nn.Module):
             if cfg.moe_norm_topk:
                 topw = topw / (topw.sum(-1, keepdim=True) + 1e-20)
             topw = topw * cfg.routed_scaling_factor
+        elif cfg.moe_routing == "softmax_bias":
+            # softmax over all experts; the choice adds the correction,
+            # the weights are the chosen scores themselves
+            scores = torch.softmax(logits.float(), dim=-1)
+            topi = (scores + self.e_score_correction_bias).topk(
+                self.top_k, dim=-1)[1]
+            topw = scores.gather(1, topi)
         elif cfg.moe_routing == "topk_softmax":
             # gpt-oss: top-k on raw logits, softmax over the selected k
             topl, topi = torch.topk(logits.float(), self.top_k, dim=-1)
@@ -203,7 +213,7 @@ class MoEMLP(nn.Module):
         act = torch.empty(pad, self.ie_local, dtype=x.dtype, device=x.device)
         ops.moe_gate_silu(act, x, self.w_gate_up, sorted_tok, offsets,
                           self.e_base, self.e_local, self.b_gate_up,
-                          self.act_mode)
+                          self.act_mode, self.act_limit)
         out32 = torch.zeros(T, H, dtype=torch.float32, device=x.device)
         ops.moe_down_scatter(out32, act, self.w_down, sorted_tok, gates,
                              offsets, self.e_base, self.e_local,
@@ -230,10 +240,7 @@ class MoEMLP(nn.Module):
             if self.act_mode == 2:
                 act = ops.relu2(h1)
             elif self.act_mode == 1:
-                g, u = h1.float().chunk(2, dim=-1)
-                g = g.clamp(max=7.0)
-                u = u.clamp(-7.0, 7.0)
-                act = ((u + 1.0) * (g * torch.sigmoid(1.702 * g))).to(x.dtype)
+                act = ops.clamped_glu(h1, self.act_limit)
             else:
                 act = ops.silu_and_mul(h1.contiguous())
             y = torch.nn.functional.linear(

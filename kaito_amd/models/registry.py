@@ -26,6 +26,7 @@ MODEL_CLASSES: Dict[str, str] = {
     "gurapel": "kaito_amd.models.gurapel:GurapelForCausalLM",
     "pokulorn": "kaito_amd.models.pokulorn:PokulornForCausalLM",
     "munerax": "kaito_amd.models.munerax:MuneraxForCausalLM",
+    "lokedra": "kaito_amd.models.lokedra:LokedraForCausalLM",
 }
 
 
@@ -44,7 +45,8 @@ def config_from_checkpoint(cfg_json: dict, name: str = "",
     """config.json dict → ModelConfig, choosing the reader by the file's
     own architecture tag."""
     from .hybrid_config import (gurapel_model_config, is_gurapel_config,
-                                is_munerax_config, is_pokulorn_config,
+                                is_lokedra_config, is_munerax_config,
+                                is_pokulorn_config, lokedra_model_config,
                                 munerax_model_config, pokulorn_model_config)
     kw = {"dtype": dtype} if dtype is not None else {}
     if is_gurapel_config(cfg_json):
@@ -53,6 +55,8 @@ def config_from_checkpoint(cfg_json: dict, name: str = "",
         return pokulorn_model_config(cfg_json, name=name, **kw)
     if is_munerax_config(cfg_json):
         return munerax_model_config(cfg_json, name=name, **kw)
+    if is_lokedra_config(cfg_json):
+        return lokedra_model_config(cfg_json, name=name, **kw)
     cfg = ModelConfig.from_hf_config(cfg_json, name=name)
     if dtype is not None:
         import dataclasses
@@ -439,3 +443,36 @@ def _tiny_munerax() -> ModelConfig:
 
 
 register(_tiny_munerax())
+
+
+def _tiny_lokedra() -> ModelConfig:
+    """A small looped stack of parallel layers (generalized delta rule,
+    latent attention with low-rank queries, chunked attention beside
+    HGRN2, routed clamped-GLU experts) for tests and smoke runs (random
+    weights)."""
+    from .hybrid_config import lokedra_model_config
+    moe = {"kind": "moe", "expert": {"ff": 48, "limit": 2.0},
+           "router": {"experts": 6, "top": 2}}
+    layers = [
+        {"type": "general_delta", "mixer": {"heads": 3, "dim": 16},
+         "mlp": moe},
+        {"type": "latent_attention", "mixer": {
+            "heads": 3, "dim": 16, "rot_dim": 8, "vdim": 24, "kv_rank": 40,
+            "q_rank": 56, "scale": 0.2, "rot": {
+                "base": 10000.0, "dims": 8, "scaling": {
+                    "factor": 4.0, "original": 64, "fast": 8.0,
+                    "slow": 1.0}}}, "mlp": moe},
+        {"type": "parallel", "mixer": {
+            "left": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 16,
+                     "conv": 3, "mask": {"size": 24}, "scale": 0.25},
+            "right": {"heads": 2, "dim": 16, "vdim": 24},
+            "left_scale": 0.8, "right_scale": 1.1}, "mlp": None},
+    ]
+    return lokedra_model_config({
+        "architecture": "Lokedra", "embedding": {"scale": 4.0},
+        "layers": layers, "loop": {"start": 1, "stop": 3, "times": 2},
+        "norm": {"eps": 1e-5}, "vocab": 512, "width": 192,
+        "max_positions": 1024}, name="tiny-lokedra-test")
+
+
+register(_tiny_lokedra())

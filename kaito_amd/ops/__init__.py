@@ -35,10 +35,12 @@ for _g, _names in {
     "mix": ("causal_conv_update "
             "qk_norm_cache_write window_attention window_attention_tiles "
             "post_norm_residual rms_norm_cast residual_add_norm "
+            "scaled_residual_add_norm token_shift "
             "clamped_glu sigmoid_mul gelu_glu relu2"),
     "latent": ("bigram_embed latent_rope_cache_write latent_attention "
                "latent_expand"),
     "delta": "gated_delta_rule rglru_scan",
+    "diag": "diag_delta_rule hgrn2_scan",
     "decay": "mlstm_scan ssd_scan",
 }.items():
     for _n in _names.split():
@@ -303,15 +305,16 @@ def moe_gate_silu(act: torch.Tensor, x: torch.Tensor,
                   w_gate_up: torch.Tensor, sorted_ids: torch.Tensor,
                   offsets: torch.Tensor, e_base: int,
                   n_local_experts: int, bias: torch.Tensor | None = None,
-                  act_mode: int = 0) -> None:
+                  act_mode: int = 0, act_limit: float = 7.0) -> None:
     """Fused MoE stage 1 (GPU only): gather rows by sorted token ids,
     gate/up grouped GEMM per expert, activation epilogue into `act`
-    (act_mode 0 = SwiGLU, 1 = gpt-oss clamped swiglu; optional
+    (act_mode 0 = SwiGLU, 1 = clamped swiglu min(g, limit)·sigmoid(1.702
+    g)·(clamp(u, ±limit) + 1); optional
     per-expert [E, 2*IE] bias; 2 = ungated squared relu with weights
     [E, IE, H])."""
     b = bias if bias is not None else         torch.empty(0, dtype=x.dtype, device=x.device)
-    _K.moe_gate_silu(act, x, w_gate_up, sorted_ids, offsets,
-                                  b, act_mode, e_base, n_local_experts)
+    _K.moe_gate_silu(act, x, w_gate_up, sorted_ids, offsets, b, act_mode,
+                     e_base, n_local_experts, act_limit)
 
 
 def moe_down_scatter(out: torch.Tensor, act: torch.Tensor,
@@ -470,11 +473,12 @@ WINDOW_MFMA_VSIZES = (32, 64, 128, 256)     # value sizes
 def window_attention(q, k_cache, v_cache, block_tables, token_seq, positions,
                      scale: float, softcap: float = 0.0, r1=None, r2=None,
                      window: int = 0, tiles=None, keep_first: int = 0,
-                     sinks=None):
+                     sinks=None, chunk: int = 0):
     """Causal attention of query rows [T, H, D] over the paged cache (key
     size D, value size V may differ). A query at position i sees keys
-    j <= i with i - j < window or j < keep_first (window <= 0: all).
-    Options: tanh score capping, the distance penalty
+    j <= i with i - j < window or j < keep_first (window <= 0: all), or,
+    with `chunk` > 0, keys j <= i of i's own block of `chunk` positions
+    counted from position 0. Options: tanh score capping, the distance penalty
     r1*ln(1 + r2*distance), and per-head `sinks` [H] f32 whose exp joins
     the softmax denominator. Returns [T, H, V].
 
@@ -494,16 +498,17 @@ def window_attention(q, k_cache, v_cache, block_tables, token_seq, positions,
             _K.window_attention_tiles(
                 out, q, k_cache, v_cache, block_tables, tile_seq, tile_qbase,
                 cu, starts, scale, softcap, _none(r1, q), _none(r2, q),
-                window, keep_first, _none(sinks, q))
+                window, keep_first, _none(sinks, q), chunk)
             return out
         _K.window_attention(out, q, k_cache, v_cache, block_tables, token_seq,
                             positions, scale, softcap, _none(r1, q),
                             _none(r2, q), window, keep_first,
-                            _none(sinks, q))
+                            _none(sinks, q), chunk)
         return out
     return torch_ref.window_attention(q, k_cache, v_cache, block_tables,
                                       token_seq, positions, scale, softcap,
-                                      r1, r2, window, keep_first, sinks)
+                                      r1, r2, window, keep_first, sinks,
+                                      chunk)
 
 
 def build_query_tiles(chunk_lens, device):
@@ -665,10 +670,12 @@ def bigram_embed(ids, embed, scale: float, table, buckets: int,
 
 
 def latent_rope_cache_write(q, dkv, norm_w, eps: float, cache, slot_mapping,
-                            positions, inv_freq, dim: int, pad_to: int = 0):
+                            positions, inv_freq, dim: int, pad_to: int = 0,
+                            interleaved: bool = False, rot_mag: float = 1.0):
     """Rotation of the last 2R dims of every head of q [T, H, dim + 2R]
-    (R = len(inv_freq); i paired with i + R; angle = position *
-    inv_freq[i] in f32) and, with dkv [T, rank + 2R] given (row stride
+    (R = len(inv_freq); i paired with i + R, or with `interleaved` 2i
+    with 2i + 1; angle = position * inv_freq[i] in f32; cos and sin times
+    rot_mag) and, with dkv [T, rank + 2R] given (row stride
     free), the latent row: RMS norm of the first rank dims with the f32
     weight norm_w, rotation of the last 2R, scatter into the paged latent
     cache [blocks, block_size, rank + 2R] at slot_mapping (negative slots
@@ -683,11 +690,12 @@ def latent_rope_cache_write(q, dkv, norm_w, eps: float, cache, slot_mapping,
                                                 device=q.device),
             norm_w if own else _none(None, q), eps,
             cache if own else torch.empty(0, dtype=q.dtype, device=q.device),
-            slot_mapping, positions, inv_freq, dim)
+            slot_mapping, positions, inv_freq, dim, interleaved, rot_mag)
         return out
     out = torch_ref.latent_rope_cache_write(q, dkv, norm_w, eps, cache,
                                             slot_mapping, positions,
-                                            inv_freq, dim)
+                                            inv_freq, dim, interleaved,
+                                            rot_mag)
     if pad_to > out.size(2):
         out = torch.nn.functional.pad(out, (0, pad_to - out.size(2)))
     return out
@@ -747,3 +755,102 @@ def latent_expand(kn, vv, lat, H: int, D: int, V: int, rank: int, Dp: int,
                       device=lat.device)
     _K.latent_expand(k_s, v_s, kn, vv, lat, H, D, V, rank)
     return k_s, v_s
+
+
+# ---- looped parallel-layer stacks (groups "mix" and "diag") -----------------
+
+def linear_f32(x, weight, bias=None):
+    """x [T, K] @ weight [N, K]^T (+ bias) with the result kept in f32.
+    Inputs in the activation dtype are multiplied exactly and summed in
+    f32, and the result is not rounded back to the activation dtype: what
+    feeds a recurrence's gates. On the GPU this is the vendor bf16 GEMM
+    with an f32 output; where the build lacks that, an f32 GEMM."""
+    global _MM_F32_OUT
+    if x.dtype != torch.float32 and x.is_cuda and _MM_F32_OUT:
+        try:
+            out = torch.mm(x, weight.t(), out_dtype=torch.float32)
+            return out if bias is None else out + bias
+        except (RuntimeError, TypeError):
+            _MM_F32_OUT = False
+    return torch.nn.functional.linear(x.float(), weight.float(), bias)
+
+
+_MM_F32_OUT = True
+
+
+def scaled_residual_add_norm(x32, terms, w, eps: float, out_dtype,
+                             x_add=None):
+    """Residual step with per-channel sub-layer scales on an f32 stream
+    [T, H]: x32 += sum of v*y over `terms`, one to three pairs (y [T, H]
+    in the activation dtype, v [H] f32), (+ x_add [T, H] f32), in place;
+    returns rms(x32)*w rounded to out_dtype, the next layer's input (None
+    when w is None)."""
+    assert 1 <= len(terms) <= 3
+    if x32.is_cuda:
+        h = torch.empty(x32.shape, dtype=out_dtype, device=x32.device) \
+            if w is not None else x32
+        y0 = terms[0][0]
+        ys = [t[0] for t in terms] + [_none(None, y0)] * (3 - len(terms))
+        vs = [t[1] for t in terms] + [_none(None, y0)] * (3 - len(terms))
+        _K.scaled_residual_add_norm(x32, h, ys[0], ys[1], ys[2], vs[0],
+                                    vs[1], vs[2], _none(x_add, y0),
+                                    _none(w, y0), eps)
+        return h if w is not None else None
+    return torch_ref.scaled_residual_add_norm(x32, terms, w, eps, out_dtype,
+                                              x_add)
+
+
+def token_shift(h, mu, state, cu_seqlens, state_slots, seq_starts,
+                token_seq):
+    """Blend of every row with the row before it: h_t + (h_{t-1} - h_t)*mu
+    (mu [H] f32). A chunk's first row takes its predecessor from state
+    [slots, H] (h's dtype; zeros at position 0), which is advanced to the
+    chunk's last row. Returns [T, H]."""
+    if h.is_cuda:
+        out = torch.empty(h.shape, dtype=h.dtype, device=h.device)
+        _K.token_shift(out, h, mu, state, cu_seqlens, state_slots,
+                       seq_starts, token_seq)
+        return out
+    return torch_ref.token_shift(h, mu, state, cu_seqlens, state_slots,
+                                 seq_starts)
+
+
+def diag_delta_rule(r, k, v, w_pre, a_pre, gate, norm_w, state, cu_seqlens,
+                    state_slots, seq_starts, decay_rate: float, k_eps: float,
+                    norm_eps: float):
+    """Generalized delta rule with a decay per key channel: r/k/v/gate
+    [T, H, D] (row strides free), w_pre/a_pre [T, H*D] f32 (decay and
+    removal-rate pre-activations), norm_w [H*D] f32, state [slots, H, D, D]
+    f32 in place. S <- diag(w) S - (a*u)(u^T S) + k v^T with u the unit
+    key, w = exp(-decay_rate*sigmoid(w_pre)), a = sigmoid(a_pre); read-out
+    S^T r divided by its RMS per head, times norm_w, times sigmoid(gate).
+    Returns [T, H*D]."""
+    if r.is_cuda:
+        T, H, D = r.shape
+        out = torch.empty(T, H * D, dtype=r.dtype, device=r.device)
+        _K.diag_delta_rule(out, r, k, v, w_pre, a_pre, gate, norm_w, state,
+                           cu_seqlens, state_slots, seq_starts, decay_rate,
+                           k_eps, norm_eps)
+        return out
+    return torch_ref.diag_delta_rule(r, k, v, w_pre, a_pre, gate, norm_w,
+                                     state, cu_seqlens, state_slots,
+                                     seq_starts, decay_rate, k_eps, norm_eps)
+
+
+def hgrn2_scan(q, v, f_pre, lower, norm_w, state, cu_seqlens, state_slots,
+               seq_starts, norm_eps: float):
+    """Linear attention with a lower-bounded forget gate that also sets
+    the write: q [T, H, D] (silu applied inside), v [T, H, V] (row strides
+    free), f_pre [T, H*D] f32, lower [H*D] f32, norm_w [V] f32, state
+    [slots, H, D, V] f32 in place. f = lower + (1 - lower) sigmoid(f_pre),
+    S <- diag(f) S + (1 - f) v^T, o = S^T silu(q), RMS-normed over V with
+    norm_w. Returns [T, H*V]."""
+    if q.is_cuda:
+        T, H, V = v.shape
+        out = torch.empty(T, H * V, dtype=q.dtype, device=q.device)
+        _K.hgrn2_scan(out, q, v, f_pre, lower, norm_w, state, cu_seqlens,
+                      state_slots, seq_starts, norm_eps)
+        return out
+    return torch_ref.hgrn2_scan(q, v, f_pre, lower, norm_w, state,
+                                cu_seqlens, state_slots, seq_starts,
+                                norm_eps)

@@ -96,9 +96,12 @@ __global__ __launch_bounds__(256) void latent_rope_cache_write_kernel(
     T* __restrict__ cache, const int64_t* __restrict__ slot_mapping,
     const int64_t* __restrict__ positions,
     const float* __restrict__ inv_freq, const int H, const int dim,
-    const int R, const int rank, const int HDo, const bool vec) {
+    const int R, const int rank, const int HDo, const bool vec,
+    const bool interleaved, const float mag) {
   const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float pos = (float)positions[t];
+  // pair i is dims (i, i + R), or (2i, 2i + 1) when interleaved
+  const int pa = interleaved ? 2 : 1, pb = interleaved ? 1 : R;
   const int items = H + (dkv != nullptr ? 1 : 0);
   const int HD = dim + 2 * R;
   constexpr int VEC = 16 / (int)sizeof(T);
@@ -121,10 +124,11 @@ __global__ __launch_bounds__(256) void latent_rope_cache_write_kernel(
       }
       for (int i = lane; i < R; i += 64) {
         const float ang = pos * inv_freq[i];
-        const float c = cosf(ang), s = sinf(ang);
-        const float u = act_ld(src + dim + i), v = act_ld(src + dim + R + i);
-        act_st(dst + dim + i, u * c - v * s);
-        act_st(dst + dim + R + i, v * c + u * s);
+        const float c = cosf(ang) * mag, s = sinf(ang) * mag;
+        const int ia = dim + i * pa, ib = ia + pb;
+        const float u = act_ld(src + ia), v = act_ld(src + ib);
+        act_st(dst + ia, u * c - v * s);
+        act_st(dst + ib, v * c + u * s);
       }
       return;
     }
@@ -140,10 +144,11 @@ __global__ __launch_bounds__(256) void latent_rope_cache_write_kernel(
       act_st(dst + d, act_ld(src + d) * inv * norm_w[d]);
     for (int i = lane; i < R; i += 64) {
       const float ang = pos * inv_freq[i];
-      const float c = cosf(ang), s = sinf(ang);
-      const float u = act_ld(src + rank + i), v = act_ld(src + rank + R + i);
-      act_st(dst + rank + i, u * c - v * s);
-      act_st(dst + rank + R + i, v * c + u * s);
+      const float c = cosf(ang) * mag, s = sinf(ang) * mag;
+      const int ia = rank + i * pa, ib = ia + pb;
+      const float u = act_ld(src + ia), v = act_ld(src + ib);
+      act_st(dst + ia, u * c - v * s);
+      act_st(dst + ib, v * c + u * s);
     }
   }
 }
@@ -592,7 +597,8 @@ void bigram_embed(at::Tensor out, at::Tensor ids, at::Tensor embed,
 void latent_rope_cache_write(at::Tensor q_out, at::Tensor q, at::Tensor dkv,
                              at::Tensor norm_w, double eps, at::Tensor cache,
                              at::Tensor slot_mapping, at::Tensor positions,
-                             at::Tensor inv_freq, int64_t dim) {
+                             at::Tensor inv_freq, int64_t dim,
+                             bool interleaved, double rot_mag) {
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && is_act_dtype(q) &&
               q.stride(2) == 1);
   const int T = q.size(0), H = q.size(1), HD = q.size(2);
@@ -639,7 +645,7 @@ void latent_rope_cache_write(at::Tensor q_out, at::Tensor q, at::Tensor dkv,
         (float)eps, own ? (act_t*)cache.data_ptr() : nullptr,
         own ? slot_mapping.data_ptr<int64_t>() : nullptr,
         positions.data_ptr<int64_t>(), inv_freq.data_ptr<float>(), H,
-        (int)dim, R, rank, HDo, vec);
+        (int)dim, R, rank, HDo, vec, interleaved, (float)rot_mag);
   });
 }
 
@@ -767,7 +773,7 @@ void latent_expand(at::Tensor k_s, at::Tensor v_s, at::Tensor kn,
 
 TORCH_LIBRARY_FRAGMENT(kaito, m) {
   m.def("bigram_embed(Tensor(a!) out, Tensor ids, Tensor embed, float scale, Tensor table, int buckets, int mul_prev, int mul_cur, Tensor(b!) prev_state, Tensor cu_seqlens, Tensor state_slots, Tensor seq_starts, Tensor token_seq) -> ()");
-  m.def("latent_rope_cache_write(Tensor(a!) q_out, Tensor q, Tensor dkv, Tensor norm_w, float eps, Tensor(b!) cache, Tensor slot_mapping, Tensor positions, Tensor inv_freq, int dim) -> ()");
+  m.def("latent_rope_cache_write(Tensor(a!) q_out, Tensor q, Tensor dkv, Tensor norm_w, float eps, Tensor(b!) cache, Tensor slot_mapping, Tensor positions, Tensor inv_freq, int dim, bool interleaved, float rot_mag) -> ()");
   m.def("latent_attention(Tensor(a!) out, Tensor q, Tensor cache, Tensor block_tables, Tensor token_seq, Tensor positions, float scale, Tensor sinks) -> ()");
   m.def("latent_expand(Tensor(a!) k_s, Tensor(b!) v_s, Tensor kn, Tensor vv, Tensor lat, int H, int D, int V, int rank) -> ()");
 }

@@ -95,12 +95,12 @@ KAITO_DEV bf16x8 frag_read(const short* __restrict__ lds, int row, int kk,
 
 KAITO_DEV float silu_f(float v) { return v / (1.f + __expf(-v)); }
 
-// act_mode 1: gpt-oss clamped swiglu — gate=min(g,7), up=clamp(u,±7),
-// (up+1) * gate*sigmoid(1.702*gate)
-KAITO_DEV float moe_act_f(int mode, float g, float u) {
+// act_mode 1: clamped swiglu — gate=min(g,limit), up=clamp(u,±limit),
+// (up+1) * gate*sigmoid(1.702*gate); gpt-oss uses limit 7
+KAITO_DEV float moe_act_f(int mode, float g, float u, float limit) {
   if (mode == 1) {
-    g = fminf(g, 7.f);
-    u = fminf(fmaxf(u, -7.f), 7.f);
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
     const float glu = g / (1.f + __expf(-1.702f * g));
     return (u + 1.f) * glu;
   }
@@ -121,7 +121,7 @@ void moe_gate_silu_kernel(
     const int* __restrict__ offsets,     // [E+1] (global expert ids)
     const short* __restrict__ bias,      // [E, 2*IE] bf16 or nullptr
     const int act_mode,
-    const int e_base, const int H, const int IE) {
+    const int e_base, const int H, const int IE, const float act_limit) {
   const int e = e_base + blockIdx.y;
   const int m0 = offsets[e] + blockIdx.x * BM;
   const int m_end = offsets[e + 1];
@@ -213,7 +213,7 @@ void moe_gate_silu_kernel(
           u += bf16_to_f32(bias[(int64_t)e * 2 * IE + IE + col]);
         }
         act[(int64_t)(m0 + row) * IE + col] =
-            f32_to_bf16(moe_act_f(act_mode, g, u));
+            f32_to_bf16(moe_act_f(act_mode, g, u, act_limit));
       }
     }
   }
@@ -305,7 +305,8 @@ void moe_down_scatter_kernel(
 void moe_gate_silu(at::Tensor act, at::Tensor x, at::Tensor w_gate_up,
                    at::Tensor sorted_ids, at::Tensor offsets,
                    at::Tensor bias, int64_t act_mode,
-                   int64_t e_base, int64_t n_local_experts) {
+                   int64_t e_base, int64_t n_local_experts,
+                   double act_limit) {
   const short* bias_ptr = nullptr;
   if (bias.numel() > 0) {
     TORCH_CHECK(bias.dtype() == at::kBFloat16 && bias.is_contiguous());
@@ -335,12 +336,12 @@ void moe_gate_silu(at::Tensor act, at::Tensor x, at::Tensor w_gate_up,
       moe_gate_silu_kernel<128, false><<<grid, block, 0, stream>>>(
           (short*)act.data_ptr(), (const short*)x.data_ptr(),
           (const short*)w_gate_up.data_ptr(), sorted_ids.data_ptr<int>(),
-          offsets.data_ptr<int>(), nullptr, 2, (int)e_base, H, IE);
+          offsets.data_ptr<int>(), nullptr, 2, (int)e_base, H, IE, 0.f);
     else
       moe_gate_silu_kernel<64, false><<<grid, block, 0, stream>>>(
           (short*)act.data_ptr(), (const short*)x.data_ptr(),
           (const short*)w_gate_up.data_ptr(), sorted_ids.data_ptr<int>(),
-          offsets.data_ptr<int>(), nullptr, 2, (int)e_base, H, IE);
+          offsets.data_ptr<int>(), nullptr, 2, (int)e_base, H, IE, 0.f);
     return;
   }
   if (BN == 128)
@@ -348,13 +349,13 @@ void moe_gate_silu(at::Tensor act, at::Tensor x, at::Tensor w_gate_up,
         (short*)act.data_ptr(), (const short*)x.data_ptr(),
         (const short*)w_gate_up.data_ptr(), sorted_ids.data_ptr<int>(),
         offsets.data_ptr<int>(), bias_ptr, (int)act_mode, (int)e_base, H,
-        IE);
+        IE, (float)act_limit);
   else
     moe_gate_silu_kernel<64><<<grid, block, 0, stream>>>(
         (short*)act.data_ptr(), (const short*)x.data_ptr(),
         (const short*)w_gate_up.data_ptr(), sorted_ids.data_ptr<int>(),
         offsets.data_ptr<int>(), bias_ptr, (int)act_mode, (int)e_base, H,
-        IE);
+        IE, (float)act_limit);
 }
 
 void moe_down_scatter(at::Tensor out, at::Tensor act, at::Tensor w_down,

@@ -5,7 +5,9 @@
 //   score(i, j) = cap * tanh(q_i . k_j * scale / cap)      (cap > 0)
 //                 - r1_h * ln(1 + r2_h * (i - j))           (r1 given)
 //   visible:      j <= i and (i - j < window or j < keep_first)
-//                 (window <= 0: every j <= i)
+//                 (window <= 0: every j <= i); or, with chunk > 0,
+//                 j <= i and floor(j / chunk) == floor(i / chunk), blocks
+//                 of `chunk` positions counted from position 0
 //   sinks:        with sink_h given, exp(sink_h) joins the softmax
 //                 denominator (no key, no value): the running maximum
 //                 starts at sink_h and the running sum at 1
@@ -158,7 +160,7 @@ __global__ void window_attention_kernel(
     const float scale, const float softcap, const float* __restrict__ r1,
     const float* __restrict__ r2, const int window, const int H, const int G,
     const int D, const int V, const int BS, const int keep_first,
-    const float* __restrict__ sinks) {
+    const float* __restrict__ sinks, const int chunk) {
   extern __shared__ float lds[];
   const int KT = blockDim.x;            // keys per tile
   float* q_s = lds;                     // [D]
@@ -176,7 +178,8 @@ __global__ void window_attention_kernel(
   }
   const int g = h / (H / G);
   const int pos = (int)positions[t];
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = chunk > 0 ? (pos / chunk) * chunk
+      : (window > 0 ? max(0, pos - window + 1) : 0);
   const int nfirst = min(keep_first, lo);       // kept keys before the window
   const int nkeys = nfirst + pos - lo + 1;
   const int* bt = block_tables + (int64_t)b * max_blocks;
@@ -271,7 +274,8 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
     const int* __restrict__ block_tables, const int max_blocks,
     const float scale, const float softcap, const float* __restrict__ r1,
     const float* __restrict__ r2, const int window, const int H, const int G,
-    const int BS, const int keep_first, const float* __restrict__ sinks) {
+    const int BS, const int keep_first, const float* __restrict__ sinks,
+    const int chunk) {
   constexpr int KK = D / 32;
   constexpr int DT = DV / 16;
   const int tile = blockIdx.x;
@@ -318,8 +322,11 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
   for (int dt = 0; dt < DT; dt++) ofrag[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int kv_end = min(kv_len, q_abs0 + q0 + WQ_TILE);
-  const int kv_begin = (window > 0 && q_abs0 + q0 - window + 1 > 0)
-      ? ((q_abs0 + q0 - window + 1) / WKV_TILE) * WKV_TILE : 0;
+  // first key any row of the tile may see: the window's start of the
+  // tile's first row, or the start of that row's chunk
+  const int vis0 = chunk > 0 ? ((q_abs0 + q0) / chunk) * chunk
+      : (window > 0 ? q_abs0 + q0 - window + 1 : 0);
+  const int kv_begin = vis0 > 0 ? (vis0 / WKV_TILE) * WKV_TILE : 0;
   // key tiles: those that hold kept first tokens, then the window's
   const int first_end =
       min((keep_first + WKV_TILE - 1) / WKV_TILE * WKV_TILE, kv_begin);
@@ -376,7 +383,8 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
         const int dist = q_abs - kvp;
         if (r1) sv -= hr1 * __logf(1.0f + hr2 * (float)max(dist, 0));
         if (dist < 0 || kvp >= kv_len || qr >= q_len ||
-            (window > 0 && dist >= window && kvp >= keep_first)) sv = -1e30f;
+            (window > 0 && dist >= window && kvp >= keep_first) ||
+            (chunk > 0 && kvp < (q_abs / chunk) * chunk)) sv = -1e30f;
         p[kt][r] = sv;
       }
 #pragma unroll
@@ -468,7 +476,7 @@ __global__ __launch_bounds__(256) void window_attention_decode_kernel(
     const float scale, const float softcap, const float* __restrict__ r1,
     const float* __restrict__ r2, const int window, const int H, const int G,
     const int D, const int V, const int BS, const int KT,
-    const int keep_first, const float* __restrict__ sinks) {
+    const int keep_first, const float* __restrict__ sinks, const int chunk) {
   constexpr int VEC = 16 / (int)sizeof(T);
   extern __shared__ float lds[];
   float* s_s = lds;                            // [RT][KT]
@@ -493,7 +501,8 @@ __global__ __launch_bounds__(256) void window_attention_decode_kernel(
     return;
   }
   const int pos = (int)positions[t];
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = chunk > 0 ? (pos / chunk) * chunk
+      : (window > 0 ? max(0, pos - window + 1) : 0);
   const int nfirst = min(keep_first, lo);       // kept keys before the window
   const int nkeys = nfirst + pos - lo + 1;
   const int* bt = block_tables + (int64_t)b * max_blocks;
@@ -677,7 +686,8 @@ void launch_decode(int nch, dim3 grid, size_t lds_bytes, hipStream_t stream,
                    const at::Tensor& token_seq, const at::Tensor& positions,
                    float scale, float softcap, const float* r1,
                    const float* r2, int window, int H, int G, int D, int V,
-                   int BS, int KT, int keep_first, const float* sinks) {
+                   int BS, int KT, int keep_first, const float* sinks,
+                   int chunk) {
 #define KAITO_WDEC(NCH_)                                                     \
   if (nch == NCH_) {                                                         \
     hipLaunchKernelGGL((window_attention_decode_kernel<T, RT, NCH_>), grid,  \
@@ -686,7 +696,7 @@ void launch_decode(int nch, dim3 grid, size_t lds_bytes, hipStream_t stream,
         (const T*)v_cache.data_ptr(), block_tables.data_ptr<int>(),          \
         (int)block_tables.size(1), token_seq.data_ptr<int>(),                \
         positions.data_ptr<int64_t>(), scale, softcap, r1, r2, window, H, G, \
-        D, V, BS, KT, keep_first, sinks);                                    \
+        D, V, BS, KT, keep_first, sinks, chunk);                             \
     return;                                                                  \
   }
   KAITO_WDEC(1) KAITO_WDEC(2) KAITO_WDEC(4)
@@ -766,11 +776,15 @@ void window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
                       at::Tensor token_seq, at::Tensor positions,
                       double scale, double softcap, at::Tensor r1,
                       at::Tensor r2, int64_t window, int64_t keep_first,
-                      at::Tensor sinks) {
+                      at::Tensor sinks, int64_t chunk) {
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() &&
               is_act_dtype(q));
   TORCH_CHECK(keep_first >= 0 && keep_first < (1 << 30));
-  const int kf = window > 0 ? (int)keep_first : 0;
+  TORCH_CHECK(chunk >= 0 && chunk < (1 << 30));
+  // a chunked mask replaces the window: the keys a row sees are at most
+  // one chunk, so tiles are sized by it
+  if (chunk > 0) window = chunk;
+  const int kf = (window > 0 && chunk == 0) ? (int)keep_first : 0;
   const bool has_sinks = sinks.numel() > 0;
   if (has_sinks) {
     KAITO_CHECK_F32(sinks);
@@ -820,22 +834,22 @@ void window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
         launch_decode<act_t, 8>(nch, grid, lds_bytes, stream0, out, q,
             k_cache, v_cache, block_tables, token_seq, positions,
             (float)scale, (float)softcap, p1, p2, (int)window, H, G, D, V,
-            BS, KT, kf, ps);
+            BS, KT, kf, ps, (int)chunk);
       else if (rt == 4)
         launch_decode<act_t, 4>(nch, grid, lds_bytes, stream0, out, q,
             k_cache, v_cache, block_tables, token_seq, positions,
             (float)scale, (float)softcap, p1, p2, (int)window, H, G, D, V,
-            BS, KT, kf, ps);
+            BS, KT, kf, ps, (int)chunk);
       else if (rt == 2)
         launch_decode<act_t, 2>(nch, grid, lds_bytes, stream0, out, q,
             k_cache, v_cache, block_tables, token_seq, positions,
             (float)scale, (float)softcap, p1, p2, (int)window, H, G, D, V,
-            BS, KT, kf, ps);
+            BS, KT, kf, ps, (int)chunk);
       else
         launch_decode<act_t, 1>(nch, grid, lds_bytes, stream0, out, q,
             k_cache, v_cache, block_tables, token_seq, positions,
             (float)scale, (float)softcap, p1, p2, (int)window, H, G, D, V,
-            BS, KT, kf, ps);
+            BS, KT, kf, ps, (int)chunk);
     });
     return;
   }
@@ -857,7 +871,7 @@ void window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
         positions.data_ptr<int64_t>(), (float)scale, (float)softcap,
         bias ? r1.data_ptr<float>() : nullptr,
         bias ? r2.data_ptr<float>() : nullptr, (int)window, H, G, D, V, BS,
-        kf, has_sinks ? sinks.data_ptr<float>() : nullptr);
+        kf, has_sinks ? sinks.data_ptr<float>() : nullptr, (int)chunk);
   });
 }
 
@@ -871,10 +885,12 @@ void window_attention_tiles(at::Tensor out, at::Tensor q, at::Tensor k_cache,
                             at::Tensor cu_seqlens, at::Tensor seq_starts,
                             double scale, double softcap, at::Tensor r1,
                             at::Tensor r2, int64_t window, int64_t keep_first,
-                            at::Tensor sinks) {
+                            at::Tensor sinks, int64_t chunk) {
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() &&
               q.dtype() == at::kBFloat16);
   TORCH_CHECK(keep_first >= 0 && keep_first < (1 << 30));
+  TORCH_CHECK(chunk >= 0 && chunk < (1 << 30));
+  if (chunk > 0) window = 0;          // a chunked mask replaces the window
   const int kf = window > 0 ? (int)keep_first : 0;
   const bool has_sinks = sinks.numel() > 0;
   if (has_sinks) {
@@ -917,7 +933,7 @@ void window_attention_tiles(at::Tensor out, at::Tensor q, at::Tensor k_cache,
         (int)block_tables.size(1), (float)scale, (float)softcap,             \
         bias ? r1.data_ptr<float>() : nullptr,                               \
         bias ? r2.data_ptr<float>() : nullptr, (int)window, H, G, BS, kf,    \
-        has_sinks ? sinks.data_ptr<float>() : nullptr);                      \
+        has_sinks ? sinks.data_ptr<float>() : nullptr, (int)chunk);          \
     return;                                                                  \
   }
   KAITO_WIN_CASE(64, 64) KAITO_WIN_CASE(64, 128) KAITO_WIN_CASE(128, 64)
@@ -932,9 +948,9 @@ void window_attention_tiles(at::Tensor out, at::Tensor q, at::Tensor k_cache,
 }  // namespace kaito
 
 TORCH_LIBRARY_FRAGMENT(kaito, m) {
-  m.def("window_attention_tiles(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor tile_seq, Tensor tile_qbase, Tensor cu_seqlens, Tensor seq_starts, float scale, float softcap, Tensor r1, Tensor r2, int window, int keep_first, Tensor sinks) -> ()");
+  m.def("window_attention_tiles(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor tile_seq, Tensor tile_qbase, Tensor cu_seqlens, Tensor seq_starts, float scale, float softcap, Tensor r1, Tensor r2, int window, int keep_first, Tensor sinks, int chunk) -> ()");
   m.def("qk_norm_cache_write(Tensor(a!) q_out, Tensor q, Tensor k, Tensor v, Tensor q_w, Tensor k_w, float eps, Tensor(b!) k_cache, Tensor(c!) v_cache, Tensor slot_mapping, Tensor positions, Tensor inv_freq, float rot_mag, Tensor v_first, float v_lambda) -> ()");
-  m.def("window_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor token_seq, Tensor positions, float scale, float softcap, Tensor r1, Tensor r2, int window, int keep_first, Tensor sinks) -> ()");
+  m.def("window_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor token_seq, Tensor positions, float scale, float softcap, Tensor r1, Tensor r2, int window, int keep_first, Tensor sinks, int chunk) -> ()");
 }
 TORCH_LIBRARY_IMPL(kaito, CUDA, m) {
   m.impl("qk_norm_cache_write", &kaito::qk_norm_cache_write);

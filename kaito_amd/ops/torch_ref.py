@@ -389,13 +389,15 @@ def qk_norm_cache_write(q, k, v, q_w, k_w, eps: float, k_cache, v_cache,
 
 def window_attention(q, k_cache, v_cache, block_tables, token_seq, positions,
                      scale: float, softcap: float, r1, r2, window: int,
-                     keep_first: int = 0, sinks=None):
+                     keep_first: int = 0, sinks=None, chunk: int = 0):
     """Causal sliding-window attention of query rows over the paged cache.
     Row t belongs to chunk token_seq[t] (its block table row) at sequence
     position positions[t] and sees keys j <= pos with pos - j < window or
     j < keep_first (window <= 0: all earlier keys). score =
     cap(q.k * scale) - r1 * ln(1 + r2 * (pos - j)). With `sinks` [H] the
-    softmax denominator also holds exp(sink_h)."""
+    softmax denominator also holds exp(sink_h). With `chunk` > 0 the mask
+    is chunked instead: keys j <= pos in pos's block of `chunk` positions
+    counted from 0."""
     T, H, D = q.shape
     G, bs, V = k_cache.size(1), k_cache.size(2), v_cache.size(3)
     rep = H // G
@@ -406,6 +408,8 @@ def window_attention(q, k_cache, v_cache, block_tables, token_seq, positions,
             continue
         p = pos_l[t]
         lo = max(0, p - window + 1) if window > 0 else 0
+        if chunk > 0:
+            lo = p // chunk * chunk
         js = torch.cat([torch.arange(0, min(keep_first, lo)),
                         torch.arange(lo, p + 1)])
         blk = block_tables[seq_l[t]].long()[js // bs]
@@ -596,17 +600,23 @@ def bigram_embed(ids, embed, scale: float, table, buckets: int,
 
 
 def latent_rope_cache_write(q, dkv, norm_w, eps: float, cache, slot_mapping,
-                            positions, inv_freq, dim: int):
+                            positions, inv_freq, dim: int,
+                            interleaved: bool = False, rot_mag: float = 1.0):
     """q [T, H, dim + 2R]: the last 2R dims of every head rotate (i paired
-    with i + R, angle = position * inv_freq[i], f32). dkv [T, rank + 2R]
+    with i + R, or with `interleaved` 2i with 2i + 1; angle = position *
+    inv_freq[i], f32; cos and sin times rot_mag). dkv [T, rank + 2R]
     (or None): the first rank dims are RMS-normed with norm_w, the last
     2R rotated, and the row is scattered into cache [blocks, block_size,
     rank + 2R] at slot_mapping (negative: skipped). Returns q rotated."""
     R = inv_freq.numel()
     ang = positions.float()[:, None] * inv_freq.float()[None, :]
-    c, s = torch.cos(ang), torch.sin(ang)
+    c, s = torch.cos(ang) * rot_mag, torch.sin(ang) * rot_mag
 
     def rot(t, cc, ss):
+        if interleaved:
+            a, b = t[..., 0::2], t[..., 1::2]
+            return torch.stack([a * cc - b * ss, b * cc + a * ss],
+                               -1).flatten(-2)
         a, b = t[..., :R], t[..., R:]
         return torch.cat([a * cc - b * ss, b * cc + a * ss], -1)
     qf = q.float()
@@ -653,3 +663,95 @@ def latent_attention(q, cache, block_tables, token_seq, positions,
             w = torch.softmax(s, -1)
         out[t] = w @ rows[:, :rank]
     return out.to(q.dtype)
+
+
+# ---- looped parallel-layer stacks ------------------------------------------
+
+def scaled_residual_add_norm(x32, terms, w, eps: float, out_dtype,
+                             x_add=None):
+    """x32 [T, H] f32 += sum of v*y over `terms` = [(y [T, H], v [H] f32)]
+    (+ x_add [T, H] f32), in place; returns rms(x32)*w rounded to
+    out_dtype (None when w is None)."""
+    add = None
+    for y, v in terms:
+        t = y.float() * v.float()
+        add = t if add is None else add + t
+    x32 += add
+    if x_add is not None:
+        x32 += x_add
+    if w is None:
+        return None
+    return (x32 * torch.rsqrt(x32.pow(2).mean(-1, keepdim=True) + eps)
+            * w.float()).to(out_dtype)
+
+
+def token_shift(h, mu, state, cu_seqlens, state_slots, seq_starts):
+    """Row t becomes h_t + (h_{t-1} - h_t)*mu, mu [H] f32; the row before a
+    chunk's first comes from state [slots, H] (zeros at position 0),
+    which is advanced in place to the chunk's last row of h."""
+    out = torch.zeros_like(h)
+    m = mu.float()
+    for r0, r1, slot, start in _chunks(cu_seqlens, state_slots, seq_starts):
+        first = state[slot].float()[None] if start > 0 else \
+            torch.zeros(1, h.size(1))
+        cur = h[r0:r1].float()
+        prev = torch.cat([first, cur[:-1]], 0)
+        out[r0:r1] = (cur + (prev - cur) * m).to(h.dtype)
+        state[slot] = h[r1 - 1].to(state.dtype)
+    return out
+
+
+def diag_delta_rule(r, k, v, w_pre, a_pre, gate, norm_w, state, cu_seqlens,
+                    state_slots, seq_starts, decay_rate: float, k_eps: float,
+                    norm_eps: float):
+    """Generalized delta rule. r/k/v/gate [T, H, D]; w_pre/a_pre [T, H*D]
+    f32 pre-activations of the decay w = exp(-decay_rate*sigmoid(w_pre))
+    and the removal rate a = sigmoid(a_pre); state [slots, H, D, D] f32 in
+    place. Per token and head, with u = k/sqrt(k.k + k_eps):
+    S <- diag(w) S - (a*u)(u^T S) + k v^T, o = S^T r; o is divided by its
+    root mean square per head, weighted by norm_w [H*D] and gated by
+    sigmoid(gate). Returns [T, H*D]."""
+    T, H, D = r.shape
+    rf, kf, vf = r.float(), k.float(), v.float()
+    w = torch.exp(-decay_rate * torch.sigmoid(w_pre.float())).view(T, H, D)
+    a = torch.sigmoid(a_pre.float()).view(T, H, D)
+    u = kf * torch.rsqrt(kf.pow(2).sum(-1, keepdim=True) + k_eps)
+    au = a * u
+    out = torch.zeros(T, H, D)
+    for r0, r1, slot, start in _chunks(cu_seqlens, state_slots, seq_starts):
+        S = state[slot].clone() if start > 0 else torch.zeros(H, D, D)
+        for t in range(r0, r1):
+            p = torch.einsum("hd,hdv->hv", u[t], S)
+            S = w[t][..., None] * S - au[t][..., None] * p[:, None, :] \
+                + kf[t][..., None] * vf[t][:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, rf[t])
+        state[slot] = S
+    out = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + norm_eps)
+    out = out.reshape(T, H * D) * norm_w.float() \
+        * torch.sigmoid(gate.float().reshape(T, H * D))
+    return out.to(r.dtype)
+
+
+def hgrn2_scan(q, v, f_pre, lower, norm_w, state, cu_seqlens, state_slots,
+               seq_starts, norm_eps: float):
+    """q [T, H, D] (pre-activation; silu applied here), v [T, H, V], f_pre
+    [T, H*D] f32, lower [H*D] f32; state [slots, H, D, V] f32 in place.
+    f = lower + (1 - lower) sigmoid(f_pre); S <- diag(f) S + (1 - f) v^T,
+    o = S^T silu(q); o is RMS-normed over V with norm_w [V]. Returns
+    [T, H*V]."""
+    T, H, D = q.shape
+    V = v.size(2)
+    qf = torch.nn.functional.silu(q.float())
+    vf = v.float()
+    lo = lower.float()
+    f = (lo + (1.0 - lo) * torch.sigmoid(f_pre.float())).view(T, H, D)
+    out = torch.zeros(T, H, V)
+    for r0, r1, slot, start in _chunks(cu_seqlens, state_slots, seq_starts):
+        S = state[slot].clone() if start > 0 else torch.zeros(H, D, V)
+        for t in range(r0, r1):
+            S = f[t][..., None] * S + (1.0 - f[t])[..., None] * vf[t][:, None]
+            out[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        state[slot] = S
+    out = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + norm_eps) \
+        * norm_w.float()
+    return out.reshape(T, H * V).to(q.dtype)
