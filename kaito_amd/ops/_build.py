@@ -47,6 +47,9 @@ GROUPS: Dict[str, List[str]] = {
     "decay": ["decay_recurrence.hip"],
     # latent attention over a paged low-rank cache, hashed bigram embedding
     "latent": ["latent_attention.hip"],
+    # matrix recurrences with a decay per state row: generalized delta
+    # rule, gated linear attention with a tied write gate
+    "diag": ["diag_delta.hip"],
 }
 
 
