@@ -60,7 +60,7 @@ def parse_args():
                         "random weights; comma-separated sizes of "
                         "kaito_amd.engine.hybrid_bench.SIZES (default all), "
                         "one JSON line per size and model; --hybrid-models "
-                        "picks from gurapel, pokulorn, swa-moe, munerax, "
+                        "picks from gurapel, pokulorn, swa-moe, munerax, lokedra, "
                         "mla-moe (the latent-attention MoE transformer)")
     p.add_argument("--hybrid-batch", type=int, default=32)
     p.add_argument("--hybrid-prompt", type=int, default=2048)

@@ -1,5 +1,5 @@
 """Prefill and decode throughput of the hybrid stacks (Gurapel, Pokulorn,
-Munerax) beside each other and beside the engine's closest homogeneous
+Munerax, Lokedra) beside each other and beside the engine's closest homogeneous
 model at equal size: a sliding-window GQA transformer with the same MoE
 feed-forward (the gpt-oss class without sinks) for the recurrent hybrids,
 the latent-attention MoE transformer (deepseek class) for Munerax. Random
@@ -138,6 +138,46 @@ def munerax_config(name: str, z: dict, max_pos: int):
         "vocab": z["vocab"], "width": z["width"]}, name=f"munerax-{name}")
 
 
+def lokedra_config(name: str, z: dict, max_pos: int):
+    """The looped parallel-layer stack at the sizes of `z`: three layers
+    (generalized delta rule, latent attention with low-rank queries,
+    chunked attention beside HGRN2) run twice, so as many layer runs as
+    the other stacks have layers. Recurrent states match the Gurapel
+    stack's (one dim x dim matrix per head), the latent layer has the
+    Munerax head layout, the chunk is the other stacks' window, the
+    experts are the same count and width."""
+    from ..models.hybrid_config import lokedra_model_config
+    a = LATENT
+    moe = {"kind": "moe", "expert": {"ff": z["ff"], "limit": 7.0},
+           "router": {"experts": z["experts"], "top": z["top"]}}
+    layers = [
+        {"type": "general_delta", "mlp": moe,
+         "mixer": {"heads": z["heads"], "dim": z["dim"]}},
+        {"type": "latent_attention", "mlp": moe, "mixer": {
+            "heads": z["heads"], "dim": a["dim"], "rot_dim": a["rot_dim"],
+            "vdim": a["vdim"], "kv_rank": a["kv_rank"],
+            "q_rank": 3 * a["kv_rank"] // 2,
+            "scale": (a["dim"] + a["rot_dim"]) ** -0.5,
+            "rot": {"base": 10000.0, "dims": a["rot_dim"], "scaling": {
+                "factor": 4.0, "original": 4096, "fast": 32.0,
+                "slow": 1.0}}}},
+        {"type": "parallel", "mlp": moe, "mixer": {
+            "left": {"heads": z["heads"], "kv_heads": z["kv_heads"],
+                     "dim": z["dim"], "vdim": z["dim"], "conv": 4,
+                     "mask": {"size": z["window"]},
+                     "scale": z["dim"] ** -0.5},
+            "right": {"heads": z["heads"], "dim": z["dim"],
+                      "vdim": z["dim"]},
+            "left_scale": 0.5, "right_scale": 0.5}},
+    ]
+    return lokedra_model_config({
+        "architecture": "Lokedra", "embedding": {"scale": 1.0},
+        "layers": layers,
+        "loop": {"start": 0, "stop": 3, "times": z["layers"] // 3},
+        "max_positions": max_pos, "norm": {"eps": 1e-5},
+        "vocab": z["vocab"], "width": z["width"]}, name=f"lokedra-{name}")
+
+
 def latent_transformer_config(name: str, z: dict, max_pos: int):
     """The engine's latent-attention MoE transformer (deepseek class) with
     the same head layout, latent rank, experts, groups and shared
@@ -216,6 +256,7 @@ def run(sizes: List[str], batch: int, prompt: int, out_tokens: int,
             mcfg = {"gurapel": hybrid_config, "pokulorn": pokulorn_config,
                     "swa-moe": transformer_config,
                     "munerax": munerax_config,
+                    "lokedra": lokedra_config,
                     "mla-moe": latent_transformer_config}[kind](
                         name, z, max_pos)
             pre, dec = _measure(mcfg, batch, prompt, out_tokens, eager)
