@@ -28,6 +28,7 @@
 // A chunk that starts at position 0 starts from S = 0 whatever its slot
 // held; slots < 0 are padding and skipped.
 #include "mix_common.h"
+#include <cstdlib>
 
 namespace kaito {
 
@@ -337,20 +338,29 @@ void launch_recurrence(hipStream_t stream, int B, int H, int D, int V,
                        int64_t v_s0, int64_t v_s1, float* state,
                        const ChunkArgs& c) {
 #define KAITO_DD_CASE(DP_, PARTS_, TT_)                                       \
-  {                                                                           \
+  if (dp == DP_ && parts == PARTS_) {                                         \
     constexpr int VB = 64 / PARTS_;                                           \
     hipLaunchKernelGGL(                                                       \
         (diag_recurrence_kernel<T, DP_, PARTS_, REMOVE, TT_>),                \
         dim3(B, H, (V + VB - 1) / VB), dim3(64), 0, stream, o, su, srd, sd,   \
         sb, sk, srb, srk, v, v_s0, v_s1, state, c.cu, c.slots, c.starts, D,   \
         H, V);                                                                \
+    return;                                                                   \
   }
-  const int dpad = padded_rows(D);
-  // the widest case halves the tile to keep both LDS buffers under 64 KB
-  if (dpad == 32) KAITO_DD_CASE(8, 4, 8)
-  else if (dpad == 64) KAITO_DD_CASE(16, 4, 8)
-  else if (dpad == 128) KAITO_DD_CASE(16, 8, 8)
-  else KAITO_DD_CASE(32, 8, 4)
+  // 32 rows per lane; a wave64 VALU instruction occupies its SIMD for four
+  // cycles and the token loop is serial, so with few (chunk, head, column
+  // group) triples the rows per lane are halved to double the waves. The
+  // widest cases halve the token tile to keep both LDS buffers under 64 KB.
+  int dp = 32, parts = padded_rows(D) / 32;
+  const int64_t waves32 = (int64_t)B * H * ((V * parts + 63) / 64);
+  // KAITO_DIAG_ROWS_PER_LANE=16|32 pins the choice (A/B runs, tests)
+  const char* pin = getenv("KAITO_DIAG_ROWS_PER_LANE");
+  const int want = pin ? atoi(pin) : (waves32 < 4096 ? 16 : 32);
+  if (want == 16) { dp = 16; parts *= 2; }
+  KAITO_DD_CASE(32, 1, 8) KAITO_DD_CASE(32, 2, 8) KAITO_DD_CASE(32, 4, 8)
+  KAITO_DD_CASE(32, 8, 4) KAITO_DD_CASE(16, 2, 8) KAITO_DD_CASE(16, 4, 8)
+  KAITO_DD_CASE(16, 8, 8) KAITO_DD_CASE(16, 16, 4)
+  TORCH_CHECK(false, "diag recurrence: no kernel for ", D, " state rows");
 #undef KAITO_DD_CASE
 }
 

@@ -158,12 +158,19 @@ def delta_oracle(parts, w_pre, a_pre, norm_w, H, D, eps, rate=math.exp(-0.5),
 
 
 @pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("rows_per_lane", ["16", "32"])
 @pytest.mark.parametrize("sizes", [(3, 8), (2, 48), (1, 100), (1, 200)])
-def test_delta_rule_portions_and_batches(mode, sizes):
+def test_delta_rule_portions_and_batches(mode, sizes, rows_per_lane,
+                                         monkeypatch):
     """Head sizes for every row tiling of the kernel (32, 64, 128 and 256
-    padded rows); two sequences cut differently in shared steps, a
-    padding chunk, slots that hold another sequence's state."""
+    padded rows, at 16 and at 32 state rows per lane: the kernel picks by
+    the step's shape, the test pins it); two sequences cut differently in
+    shared steps, a padding chunk, slots that hold another sequence's
+    state."""
+    monkeypatch.setenv("KAITO_DIAG_ROWS_PER_LANE", rows_per_lane)
     dev, dt = mode
+    if dev == "cpu" and rows_per_lane == "32":
+        pytest.skip("the reference op has no tiling")
     H, D = sizes
     rng = np.random.default_rng(D)
     eps = 1e-5
@@ -255,9 +262,14 @@ def test_delta_rule_keeps_a_far_token(mode):
 # ---- HGRN2 ---------------------------------------------------------------------
 
 @pytest.mark.parametrize("mode", MODES)
-@pytest.mark.parametrize("sizes", [(3, 8, 20), (2, 32, 64), (1, 72, 9)])
-def test_hgrn2_portions_and_batches(mode, sizes):
+@pytest.mark.parametrize("rows_per_lane", ["16", "32"])
+@pytest.mark.parametrize("sizes", [(3, 8, 20), (2, 32, 64), (1, 72, 9),
+                                   (1, 130, 70)])
+def test_hgrn2_portions_and_batches(mode, sizes, rows_per_lane, monkeypatch):
+    monkeypatch.setenv("KAITO_DIAG_ROWS_PER_LANE", rows_per_lane)
     dev, dt = mode
+    if dev == "cpu" and rows_per_lane == "32":
+        pytest.skip("the reference op has no tiling")
     H, D, V = sizes
     rng = np.random.default_rng(V)
     eps, width = 1e-5, 24
