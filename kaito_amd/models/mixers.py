@@ -676,14 +676,13 @@ class DiagDeltaMixer(nn.Module):
         p = F.linear(x, self.in_proj)
         gp = ops.linear_f32(x, self.gate_proj)               # [T, n + rank]
         w_pre = F.linear(torch.tanh(gp[:, n:]), self.w2, self.w0)
-        a_pre = gp[:, :n] + self.a_bias
         hd = (s.heads, s.dim)
         o = ops.diag_delta_rule(
             p[:, :n].unflatten(-1, hd), p[:, n:2 * n].unflatten(-1, hd),
-            p[:, 2 * n:3 * n].unflatten(-1, hd), w_pre, a_pre,
+            p[:, 2 * n:3 * n].unflatten(-1, hd), w_pre, gp[:, :n],
             p[:, 3 * n:].unflatten(-1, hd), self.out_norm, cache["ssm"],
             meta.cu_seqlens, meta.state_slots, meta.seq_starts,
-            s.decay_rate, s.k_eps, self.norm_eps)
+            s.decay_rate, s.k_eps, self.norm_eps, a_bias=self.a_bias)
         return F.linear(o, self.o_proj)
 
 
@@ -720,10 +719,11 @@ class HGRN2Mixer(nn.Module):
     def forward(self, x, positions, cache, meta):
         s = self.spec
         p = F.linear(x, self.in_proj)
-        f_pre = ops.linear_f32(x, self.f_proj, self.f_bias)
+        f_pre = ops.linear_f32(x, self.f_proj)
         o = ops.hgrn2_scan(
             p[:, :self.n_q].unflatten(-1, (s.heads, s.dim)),
             p[:, self.n_q:].unflatten(-1, (s.heads, s.vdim)), f_pre,
             self.lower, self.out_norm, cache["ssm"], meta.cu_seqlens,
-            meta.state_slots, meta.seq_starts, self.norm_eps)
+            meta.state_slots, meta.seq_starts, self.norm_eps,
+            f_bias=self.f_bias)
         return F.linear(o, self.o_proj)

@@ -817,40 +817,44 @@ def token_shift(h, mu, state, cu_seqlens, state_slots, seq_starts,
 
 def diag_delta_rule(r, k, v, w_pre, a_pre, gate, norm_w, state, cu_seqlens,
                     state_slots, seq_starts, decay_rate: float, k_eps: float,
-                    norm_eps: float):
+                    norm_eps: float, a_bias=None):
     """Generalized delta rule with a decay per key channel: r/k/v/gate
     [T, H, D] (row strides free), w_pre/a_pre [T, H*D] f32 (decay and
     removal-rate pre-activations), norm_w [H*D] f32, state [slots, H, D, D]
     f32 in place. S <- diag(w) S - (a*u)(u^T S) + k v^T with u the unit
-    key, w = exp(-decay_rate*sigmoid(w_pre)), a = sigmoid(a_pre); read-out
-    S^T r divided by its RMS per head, times norm_w, times sigmoid(gate).
-    Returns [T, H*D]."""
+    key, w = exp(-decay_rate*sigmoid(w_pre)), a = sigmoid(a_pre + a_bias)
+    (a_bias [H*D] f32, optional); read-out S^T r divided by its RMS per
+    head, times norm_w, times sigmoid(gate). Returns [T, H*D]."""
     if r.is_cuda:
         T, H, D = r.shape
         out = torch.empty(T, H * D, dtype=r.dtype, device=r.device)
-        _K.diag_delta_rule(out, r, k, v, w_pre, a_pre, gate, norm_w, state,
-                           cu_seqlens, state_slots, seq_starts, decay_rate,
-                           k_eps, norm_eps)
+        _K.diag_delta_rule(out, r, k, v, w_pre, a_pre, _none(a_bias, r), gate,
+                           norm_w, state, cu_seqlens, state_slots, seq_starts,
+                           decay_rate, k_eps, norm_eps)
         return out
+    if a_bias is not None:
+        a_pre = a_pre + a_bias
     return torch_ref.diag_delta_rule(r, k, v, w_pre, a_pre, gate, norm_w,
                                      state, cu_seqlens, state_slots,
                                      seq_starts, decay_rate, k_eps, norm_eps)
 
 
 def hgrn2_scan(q, v, f_pre, lower, norm_w, state, cu_seqlens, state_slots,
-               seq_starts, norm_eps: float):
+               seq_starts, norm_eps: float, f_bias=None):
     """Linear attention with a lower-bounded forget gate that also sets
     the write: q [T, H, D] (silu applied inside), v [T, H, V] (row strides
     free), f_pre [T, H*D] f32, lower [H*D] f32, norm_w [V] f32, state
-    [slots, H, D, V] f32 in place. f = lower + (1 - lower) sigmoid(f_pre),
-    S <- diag(f) S + (1 - f) v^T, o = S^T silu(q), RMS-normed over V with
+    [slots, H, D, V] f32 in place. f = lower + (1 - lower) sigmoid(f_pre +
+    f_bias) (f_bias [H*D] f32, optional), S <- diag(f) S + (1 - f) v^T, o = S^T silu(q), RMS-normed over V with
     norm_w. Returns [T, H*V]."""
     if q.is_cuda:
         T, H, V = v.shape
         out = torch.empty(T, H * V, dtype=q.dtype, device=q.device)
-        _K.hgrn2_scan(out, q, v, f_pre, lower, norm_w, state, cu_seqlens,
-                      state_slots, seq_starts, norm_eps)
+        _K.hgrn2_scan(out, q, v, f_pre, _none(f_bias, q), lower, norm_w,
+                      state, cu_seqlens, state_slots, seq_starts, norm_eps)
         return out
+    if f_bias is not None:
+        f_pre = f_pre + f_bias
     return torch_ref.hgrn2_scan(q, v, f_pre, lower, norm_w, state,
                                 cu_seqlens, state_slots, seq_starts,
                                 norm_eps)

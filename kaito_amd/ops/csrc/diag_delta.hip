@@ -3,10 +3,11 @@
 //
 //   diag_delta_rule   S <- diag(w) S - (a*u)(u^T S) + k v^T,   o = S^T r
 //                     u = k / sqrt(k.k + eps), w = exp(-rate*sigmoid(w_pre)),
-//                     a = sigmoid(a_pre); o / rms(o) per head, times a
+//                     a = sigmoid(a_pre + a_bias); o / rms(o) per head, times a
 //                     weight over all heads, times sigmoid(gate)
 //   hgrn2_scan        S <- diag(f) S + (1 - f) v^T,            o = S^T q
-//                     f = lower + (1 - lower) sigmoid(f_pre), q = silu(q_pre);
+//                     f = lower + (1 - lower) sigmoid(f_pre + f_bias),
+//                     q = silu(q_pre);
 //                     rms(o) over the value size with a shared weight
 //
 // Per head the state S is [D, V] f32 in a slot of its sequence. Both are
@@ -47,6 +48,7 @@ __global__ __launch_bounds__(64) void diag_delta_prep_kernel(
     const T* __restrict__ k, const int64_t k_s0, const int64_t k_s1,
     const float* __restrict__ w_pre, const int64_t w_s0,
     const float* __restrict__ a_pre, const int64_t a_s0,
+    const float* __restrict__ a_bias,                     // [H*D] or null
     const int H, const int D, const int DPAD, const float rate,
     const float k_eps) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -54,6 +56,7 @@ __global__ __launch_bounds__(64) void diag_delta_prep_kernel(
   const T* kr = k + (int64_t)t * k_s0 + (int64_t)h * k_s1;
   const float* wr = w_pre + (int64_t)t * w_s0 + (int64_t)h * D;
   const float* ar = a_pre + (int64_t)t * a_s0 + (int64_t)h * D;
+  const float* abr = a_bias ? a_bias + (int64_t)h * D : nullptr;
   float ss = 0.f;
   for (int i = lane; i < D; i += 64) {
     const float kv = act_ld(kr + i);
@@ -70,7 +73,7 @@ __global__ __launch_bounds__(64) void diag_delta_prep_kernel(
       const float rv = act_ld(rr + i);
       u = kv * inv;
       d = expf(-rate * sigmoid_f(wr[i]));
-      b = sigmoid_f(ar[i]) * u;
+      b = sigmoid_f(ar[i] + (abr ? abr[i] : 0.f)) * u;
       rd = rv * d;
       rb += rv * b;
       rk += rv * kv;
@@ -93,19 +96,21 @@ __global__ __launch_bounds__(64) void hgrn2_prep_kernel(
     float* __restrict__ srk,
     const T* __restrict__ q, const int64_t q_s0, const int64_t q_s1,
     const float* __restrict__ f_pre, const int64_t f_s0,
+    const float* __restrict__ f_bias,                     // [H*D] or null
     const float* __restrict__ lower, const int H, const int D,
     const int DPAD) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const T* qr = q + (int64_t)t * q_s0 + (int64_t)h * q_s1;
   const float* fr = f_pre + (int64_t)t * f_s0 + (int64_t)h * D;
   const float* lr = lower + (int64_t)h * D;
+  const float* fbr = f_bias ? f_bias + (int64_t)h * D : nullptr;
   const int64_t o = ((int64_t)t * H + h) * DPAD;
   float rk = 0.f;
   for (int i = lane; i < DPAD; i += 64) {
     float rd = 0.f, d = 0.f, kv = 0.f;
     if (i < D) {
       const float lo = lr[i];
-      d = lo + (1.0f - lo) * sigmoid_f(fr[i]);
+      d = lo + (1.0f - lo) * sigmoid_f(fr[i] + (fbr ? fbr[i] : 0.f));
       kv = 1.0f - d;
       const float qv = silu_f(act_ld(qr + i));
       rd = qv * d;
@@ -367,8 +372,8 @@ void launch_recurrence(hipStream_t stream, int B, int H, int D, int V,
 }  // namespace
 
 void diag_delta_rule(at::Tensor out, at::Tensor r, at::Tensor k, at::Tensor v,
-                     at::Tensor w_pre, at::Tensor a_pre, at::Tensor gate,
-                     at::Tensor norm_w, at::Tensor state, at::Tensor cu_seqlens,
+                     at::Tensor w_pre, at::Tensor a_pre, at::Tensor a_bias,
+                     at::Tensor gate, at::Tensor norm_w, at::Tensor state, at::Tensor cu_seqlens,
                      at::Tensor state_slots, at::Tensor seq_starts,
                      double decay_rate, double k_eps, double norm_eps) {
   TORCH_CHECK(r.is_cuda() && r.dim() == 3 && is_act_dtype(r));
@@ -384,6 +389,8 @@ void diag_delta_rule(at::Tensor out, at::Tensor r, at::Tensor k, at::Tensor v,
                 "gate pre-activations: f32 [T, heads*dim]");
   };
   check_pre(w_pre); check_pre(a_pre);
+  const bool ab = a_bias.numel() > 0;
+  if (ab) { KAITO_CHECK_F32(a_bias); TORCH_CHECK(a_bias.numel() == H * D); }
   KAITO_CHECK_F32(norm_w); KAITO_CHECK_F32(state);
   TORCH_CHECK(norm_w.numel() == H * D);
   TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == D &&
@@ -409,7 +416,8 @@ void diag_delta_rule(at::Tensor out, at::Tensor r, at::Tensor k, at::Tensor v,
         (const act_t*)r.data_ptr(), r.stride(0), r.stride(1),
         (const act_t*)k.data_ptr(), k.stride(0), k.stride(1),
         w_pre.data_ptr<float>(), w_pre.stride(0), a_pre.data_ptr<float>(),
-        a_pre.stride(0), H, D, DPAD, (float)decay_rate, (float)k_eps);
+        a_pre.stride(0), ab ? a_bias.data_ptr<float>() : nullptr, H, D, DPAD,
+        (float)decay_rate, (float)k_eps);
     launch_recurrence<act_t, true>(stream, c.B, H, D, D,
         o.data_ptr<float>(), su, srd, sd, sb, sk, srb, srk,
         (const act_t*)v.data_ptr(), v.stride(0), v.stride(1),
@@ -422,7 +430,7 @@ void diag_delta_rule(at::Tensor out, at::Tensor r, at::Tensor k, at::Tensor v,
 }
 
 void hgrn2_scan(at::Tensor out, at::Tensor q, at::Tensor v, at::Tensor f_pre,
-                at::Tensor lower, at::Tensor norm_w, at::Tensor state,
+                at::Tensor f_bias, at::Tensor lower, at::Tensor norm_w, at::Tensor state,
                 at::Tensor cu_seqlens, at::Tensor state_slots,
                 at::Tensor seq_starts, double norm_eps) {
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && is_act_dtype(q) &&
@@ -437,6 +445,8 @@ void hgrn2_scan(at::Tensor out, at::Tensor q, at::Tensor v, at::Tensor f_pre,
               "gate pre-activations: f32 [T, heads*dim]");
   KAITO_CHECK_F32(lower); KAITO_CHECK_F32(norm_w); KAITO_CHECK_F32(state);
   TORCH_CHECK(lower.numel() == H * D && norm_w.numel() == V);
+  const bool fb = f_bias.numel() > 0;
+  if (fb) { KAITO_CHECK_F32(f_bias); TORCH_CHECK(f_bias.numel() == H * D); }
   TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == D &&
               state.size(3) == V);
   TORCH_CHECK(out.is_contiguous() && out.dtype() == q.dtype() &&
@@ -457,7 +467,8 @@ void hgrn2_scan(at::Tensor out, at::Tensor q, at::Tensor v, at::Tensor f_pre,
     hipLaunchKernelGGL((hgrn2_prep_kernel<act_t>), dim3(T, H), dim3(64), 0,
         stream, srd, sd, sk, srk, (const act_t*)q.data_ptr(), q.stride(0),
         q.stride(1), f_pre.data_ptr<float>(), f_pre.stride(0),
-        lower.data_ptr<float>(), H, D, DPAD);
+        fb ? f_bias.data_ptr<float>() : nullptr, lower.data_ptr<float>(), H,
+        D, DPAD);
     launch_recurrence<act_t, false>(stream, c.B, H, D, V,
         o.data_ptr<float>(), nullptr, srd, sd, nullptr, sk, nullptr, srk,
         (const act_t*)v.data_ptr(), v.stride(0), v.stride(1),
@@ -472,8 +483,8 @@ void hgrn2_scan(at::Tensor out, at::Tensor q, at::Tensor v, at::Tensor f_pre,
 }  // namespace kaito
 
 TORCH_LIBRARY_FRAGMENT(kaito, m) {
-  m.def("diag_delta_rule(Tensor(a!) out, Tensor r, Tensor k, Tensor v, Tensor w_pre, Tensor a_pre, Tensor gate, Tensor norm_w, Tensor(b!) state, Tensor cu_seqlens, Tensor state_slots, Tensor seq_starts, float decay_rate, float k_eps, float norm_eps) -> ()");
-  m.def("hgrn2_scan(Tensor(a!) out, Tensor q, Tensor v, Tensor f_pre, Tensor lower, Tensor norm_w, Tensor(b!) state, Tensor cu_seqlens, Tensor state_slots, Tensor seq_starts, float norm_eps) -> ()");
+  m.def("diag_delta_rule(Tensor(a!) out, Tensor r, Tensor k, Tensor v, Tensor w_pre, Tensor a_pre, Tensor a_bias, Tensor gate, Tensor norm_w, Tensor(b!) state, Tensor cu_seqlens, Tensor state_slots, Tensor seq_starts, float decay_rate, float k_eps, float norm_eps) -> ()");
+  m.def("hgrn2_scan(Tensor(a!) out, Tensor q, Tensor v, Tensor f_pre, Tensor f_bias, Tensor lower, Tensor norm_w, Tensor(b!) state, Tensor cu_seqlens, Tensor state_slots, Tensor seq_starts, float norm_eps) -> ()");
 }
 TORCH_LIBRARY_IMPL(kaito, CUDA, m) {
   m.impl("diag_delta_rule", &kaito::diag_delta_rule);
