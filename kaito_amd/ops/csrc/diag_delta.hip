@@ -342,9 +342,10 @@ void launch_recurrence(hipStream_t stream, int B, int H, int D, int V,
                        const float* srb, const float* srk, const T* v,
                        int64_t v_s0, int64_t v_s1, float* state,
                        const ChunkArgs& c) {
-#define KAITO_DD_CASE(DP_, PARTS_, TT_)                                       \
+#define KAITO_DD_CASE(DP_, PARTS_, TTR_, TTP_)                                \
   if (dp == DP_ && parts == PARTS_) {                                         \
     constexpr int VB = 64 / PARTS_;                                           \
+    constexpr int TT_ = REMOVE ? TTR_ : TTP_;                                 \
     hipLaunchKernelGGL(                                                       \
         (diag_recurrence_kernel<T, DP_, PARTS_, REMOVE, TT_>),                \
         dim3(B, H, (V + VB - 1) / VB), dim3(64), 0, stream, o, su, srd, sd,   \
@@ -354,17 +355,21 @@ void launch_recurrence(hipStream_t stream, int B, int H, int D, int V,
   }
   // 32 rows per lane; a wave64 VALU instruction occupies its SIMD for four
   // cycles and the token loop is serial, so with few (chunk, head, column
-  // group) triples the rows per lane are halved to double the waves. The
-  // widest cases halve the token tile to keep both LDS buffers under 64 KB.
+  // group) triples the rows per lane are halved to double the waves.
+  // Tokens per tile (with / without the removal term, which stages five
+  // instead of three rows per token): as many as keep both LDS buffers of
+  // a single-wave workgroup small enough for a CU to hold at least four
+  // (one per SIMD); decode-sized steps take the shortest tile.
   int dp = 32, parts = padded_rows(D) / 32;
   const int64_t waves32 = (int64_t)B * H * ((V * parts + 63) / 64);
   // KAITO_DIAG_ROWS_PER_LANE=16|32 pins the choice (A/B runs, tests)
   const char* pin = getenv("KAITO_DIAG_ROWS_PER_LANE");
   const int want = pin ? atoi(pin) : (waves32 < 4096 ? 16 : 32);
   if (want == 16) { dp = 16; parts *= 2; }
-  KAITO_DD_CASE(32, 1, 8) KAITO_DD_CASE(32, 2, 8) KAITO_DD_CASE(32, 4, 8)
-  KAITO_DD_CASE(32, 8, 4) KAITO_DD_CASE(16, 2, 8) KAITO_DD_CASE(16, 4, 8)
-  KAITO_DD_CASE(16, 8, 8) KAITO_DD_CASE(16, 16, 4)
+  KAITO_DD_CASE(32, 1, 8, 8) KAITO_DD_CASE(32, 2, 4, 4)
+  KAITO_DD_CASE(32, 4, 2, 2) KAITO_DD_CASE(32, 8, 1, 1)
+  KAITO_DD_CASE(16, 2, 8, 8) KAITO_DD_CASE(16, 4, 8, 8)
+  KAITO_DD_CASE(16, 8, 6, 8) KAITO_DD_CASE(16, 16, 3, 4)
   TORCH_CHECK(false, "diag recurrence: no kernel for ", D, " state rows");
 #undef KAITO_DD_CASE
 }
