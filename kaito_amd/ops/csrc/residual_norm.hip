@@ -117,7 +117,9 @@ __global__ void residual_add_norm_kernel(
     act_st(h_out + (int64_t)row * H + i, xr[i] * inv * w[i]);
 }
 
-template <typename T, typename TO>
+// N = number of (y, v) terms, known at compile time so that the row loop
+// has no branches and its loads are issued together
+template <typename T, typename TO, int N>
 __global__ void scaled_residual_add_norm_kernel(
     float* __restrict__ x32, TO* __restrict__ h_out,
     const T* __restrict__ y0, const int64_t s0, const T* __restrict__ y1,
@@ -129,14 +131,14 @@ __global__ void scaled_residual_add_norm_kernel(
   const int row = blockIdx.x;
   float* xr = x32 + (int64_t)row * H;
   const T* r0 = y0 + (int64_t)row * s0;
-  const T* r1 = y1 ? y1 + (int64_t)row * s1 : nullptr;
-  const T* r2 = y2 ? y2 + (int64_t)row * s2 : nullptr;
+  const T* r1 = N > 1 ? y1 + (int64_t)row * s1 : nullptr;
+  const T* r2 = N > 2 ? y2 + (int64_t)row * s2 : nullptr;
   const float* ar = x_add ? x_add + (int64_t)row * H : nullptr;
   float ss = 0.f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float add = v0[i] * act_ld(r0 + i);
-    if (r1) add += v1[i] * act_ld(r1 + i);
-    if (r2) add += v2[i] * act_ld(r2 + i);
+    if constexpr (N > 1) add += v1[i] * act_ld(r1 + i);
+    if constexpr (N > 2) add += v2[i] * act_ld(r2 + i);
     float v = xr[i] + add;
     if (ar) v += ar[i];
     xr[i] = v;
@@ -327,9 +329,10 @@ void scaled_residual_add_norm(at::Tensor x32, at::Tensor h_out, at::Tensor y0,
   const int threads = row_threads(H);
   KAITO_DISPATCH_ACT(y0, {
     using in_t = act_t;
-    auto launch = [&](auto* ho) {
+    auto launch_n = [&](auto* ho, auto nterms) {
       using out_t = std::remove_pointer_t<decltype(ho)>;
-      hipLaunchKernelGGL((scaled_residual_add_norm_kernel<in_t, out_t>),
+      constexpr int N = decltype(nterms)::value;
+      hipLaunchKernelGGL((scaled_residual_add_norm_kernel<in_t, out_t, N>),
           dim3(T), dim3(threads), 0, stream, x32.data_ptr<float>(), ho,
           (const in_t*)y0.data_ptr(), y0.stride(0),
           t1 ? (const in_t*)y1.data_ptr() : nullptr, t1 ? y1.stride(0) : 0,
@@ -338,6 +341,11 @@ void scaled_residual_add_norm(at::Tensor x32, at::Tensor h_out, at::Tensor y0,
           t2 ? v2.data_ptr<float>() : nullptr,
           addx ? x_add.data_ptr<float>() : nullptr,
           norm ? w.data_ptr<float>() : nullptr, H, (float)eps);
+    };
+    auto launch = [&](auto* ho) {
+      if (t2) launch_n(ho, std::integral_constant<int, 3>{});
+      else if (t1) launch_n(ho, std::integral_constant<int, 2>{});
+      else launch_n(ho, std::integral_constant<int, 1>{});
     };
     if (norm && h_out.dtype() == at::kBFloat16)
       launch((bf16_act*)h_out.data_ptr());
