@@ -422,7 +422,7 @@ def test_catalog_resolves_checkpoint_folder(tmp_path_factory):
     assert s3.ddelta.dim == 72 and s3.ddelta.heads == 1
     assert resolve_model_class(mc).__name__ == "LokedraForCausalLM"
     ca = checkpoint(tmp_path_factory, "a")[2]
-    lp = get_model_config("another", weights_path=ca).layer_loop
+    lp = get_model_config("another-looped-stack", weights_path=ca).layer_loop
     assert (lp.start, lp.stop, lp.times) == (1, 3, 3)
 
 
