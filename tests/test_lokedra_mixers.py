@@ -620,3 +620,22 @@ def test_routed_clamped_experts(mode, sizes):
             / np.abs(want).max()
         assert err.median().item() < 2e-2
         assert (err < 4e-2).float().mean() > 0.8
+
+
+# ---- projections whose result stays f32 ---------------------------------------------
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("shape", [(37, 96, 50), (5, 72, 33), (128, 256, 192)])
+def test_gate_projection_keeps_f32(mode, shape):
+    """bf16 operands multiply exactly; the sum must not be rounded back to
+    bf16 (a sigmoid near 0 or 1 would lose its tail)."""
+    dev, dt = mode
+    T, K, N = shape
+    rng = np.random.default_rng(T)
+    x, xf = act(rng.normal(0, 1, (T, K)), mode)
+    w, wf = act(rng.normal(0, 1, (N, K)), mode)
+    b = rng.normal(0, 1, N)
+    got = ops.linear_f32(x, w, torch.tensor(b, dtype=torch.float32,
+                                            device=dev))
+    assert got.dtype == torch.float32
+    close(got, xf @ wf.T + np.float32(b), torch.float32, f32=2e-6)
