@@ -141,7 +141,7 @@ class RotaryAttnSpec:
     gate: bool = False
     qk_norm: bool = True
     # a chunked mask instead of a window: query i sees j <= i only with
-    # floor(i / chunk) == floor(j / chunk), chunks counted from position 0
+    # floor(i / chunk) == floor(j / chunk) on absolute sequence positions
     chunk: int = 0
     bias: bool = False            # biases on the q/k/v and output projections
     tied_values: bool = False     # no value projection: v = k as cached
@@ -233,9 +233,10 @@ class HGRN2Spec:
 
 @dataclass(frozen=True)
 class LoopSpec:
-    """Layers start .. stop-1 run `times` times in a row with the same
-    weights (each pass with caches and states of its own); before every
-    pass but the first the embedding output is added to the stream."""
+    """A repeated block: layers [start, stop) execute `times` passes back
+    to back on shared weights, each pass keeping caches and states of its
+    own; from the second pass on, a pass opens with x += the embedding
+    output."""
     start: int
     stop: int
     times: int
@@ -579,7 +580,7 @@ def _lokedra_layer(entry: dict) -> LayerSpec:
     if kind == "parallel":
         lf, rt = mx["left"], mx["right"]
         if int(lf.get("vdim", lf["dim"])) != int(lf["dim"]):
-            raise ValueError("values are the keys: vdim must equal dim")
+            raise ValueError("keys double as values: vdim must equal dim")
         mask = lf.get("mask") or {}
         return LayerSpec(
             kind,

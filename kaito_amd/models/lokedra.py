@@ -17,10 +17,10 @@ HGRN2Mixer — summed with config weights. The feed-forward is the
 engine's MoEMLP with clamped-GLU experts and softmax routing whose choice
 carries a per-expert correction.
 
-A run of layers may be executed several times with the same weights
-(LoopSpec): every execution ("run") of a layer has caches and states of
-its own, and before every pass but the first the embedding output is
-added to the stream. Output: the model's norm, then the embedding table
+A block of layers may be repeated on shared weights (LoopSpec): every
+execution ("run") of a layer keeps caches and states of its own, and from
+the second pass on a pass opens by adding the embedding output back
+into the stream. Output: the model's norm, then the embedding table
 as the head.
 
 The residual add of a layer is fused with the norm of the next run

@@ -687,10 +687,10 @@ class DiagDeltaMixer(nn.Module):
 
 
 class HGRN2Mixer(nn.Module):
-    """Gated linear attention in which the forget gate also decides what
-    is written: per head S <- diag(f) S + (1 - f) v^T, o = S^T q with
+    """Gated linear attention with one gate for forgetting and writing (a
+    channel that keeps a fraction f takes in 1 - f): per head S <- diag(f) S + (1 - f) v^T, o = S^T q with
     q = silu(W_q x) and f = lower + (1 - lower) sigmoid(W_f x + b) per head
-    and channel (f acts on the state rows that belong to q's channels).
+    and channel (f scales state rows, which are indexed like q).
     o is RMS-normed over vdim with a weight shared by the heads and
     projected out. The gate pre-activation stays f32."""
 

@@ -477,8 +477,8 @@ def window_attention(q, k_cache, v_cache, block_tables, token_seq, positions,
     """Causal attention of query rows [T, H, D] over the paged cache (key
     size D, value size V may differ). A query at position i sees keys
     j <= i with i - j < window or j < keep_first (window <= 0: all), or,
-    with `chunk` > 0, keys j <= i of i's own block of `chunk` positions
-    counted from position 0. Options: tanh score capping, the distance penalty
+    with `chunk` > 0, keys j <= i of i's own block of `chunk` absolute
+    positions (block b = positions [b*chunk, (b+1)*chunk)). Options: tanh score capping, the distance penalty
     r1*ln(1 + r2*distance), and per-head `sinks` [H] f32 whose exp joins
     the softmax denominator. Returns [T, H, V].
 

@@ -6,8 +6,8 @@
 //                 - r1_h * ln(1 + r2_h * (i - j))           (r1 given)
 //   visible:      j <= i and (i - j < window or j < keep_first)
 //                 (window <= 0: every j <= i); or, with chunk > 0,
-//                 j <= i and floor(j / chunk) == floor(i / chunk), blocks
-//                 of `chunk` positions counted from position 0
+//                 j <= i and floor(j / chunk) == floor(i / chunk) on
+//                 absolute sequence positions
 //   sinks:        with sink_h given, exp(sink_h) joins the softmax
 //                 denominator (no key, no value): the running maximum
 //                 starts at sink_h and the running sum at 1

@@ -217,7 +217,7 @@ def moe_ff(h, W, pre, mlp):
 
 def layer_runs(cfg):
     """Layer indices in execution order, with True where the embedding
-    output is added first (start of every loop pass but the first)."""
+    output is added first (the opening of the second and later passes)."""
     n = len(cfg["layers"])
     lp = cfg.get("loop")
     if not lp:

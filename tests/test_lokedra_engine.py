@@ -433,7 +433,7 @@ def test_config_reader_rejects_bad_files():
     with pytest.raises(ValueError):
         lokedra_model_config(cfg)
     cfg = config_a()
-    cfg["layers"][0]["mixer"]["left"]["vdim"] = 4   # values are the keys
+    cfg["layers"][0]["mixer"]["left"]["vdim"] = 4   # keys double as values
     with pytest.raises(ValueError):
         lokedra_model_config(cfg)
     cfg = config_a()
